@@ -1,0 +1,218 @@
+/*
+ * sar.h -- C ABI of the MI355X (gfx950) executor for emulated n-rank
+ * AllReduce schedules (StragglAR, ring, recursive halving/doubling, direct).
+ *
+ * All emulated ranks live in one GPU's HBM; a schedule round becomes one
+ * batched kernel launch of fused chunk moves and reduces.  The reference has
+ * no library boundary for this path: its executors are functions inside a
+ * single benchmark translation unit.  Each entry point below therefore names
+ * the reference function (file:line under the reference checkout) whose role
+ * it takes over.
+ *
+ * Conventions: every function returns 0 on success or a negative SAR_E*
+ * code; sar_last_error() gives a thread-local message for the last failure on
+ * the calling thread.  No exceptions cross the boundary.  A context is used
+ * by one host thread at a time.  The caller owns host memory, the context
+ * owns device memory.  There is no CPU fallback: without a usable HIP device
+ * sar_create() fails.
+ */
+#ifndef SAR_H
+#define SAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SAR_VERSION 100
+
+enum {
+    SAR_OK = 0,
+    SAR_EINVAL = -1,      /* bad argument */
+    SAR_ENODEV = -2,      /* no usable HIP device */
+    SAR_ENOMEM = -3,      /* host or device allocation failed */
+    SAR_EHIP = -4,        /* a HIP runtime call failed */
+    SAR_EPARSE = -5,      /* schedule text not understood */
+    SAR_ESCHED = -6,      /* schedule is not valid */
+    SAR_ESTATE = -7       /* call made in the wrong state (e.g. run before prepare) */
+};
+
+enum { SAR_F32 = 0, SAR_F16 = 1, SAR_BF16 = 2 };
+
+/* operation kinds of the schedule representation (one row of a round) */
+enum {
+    SAR_OP_COPY = 0,        /* dst chunk <- src chunk                       (a plain ncclSend/ncclRecv pair)        */
+    SAR_OP_XREDUCE = 1,     /* s = a + b; a <- s; b <- s                    (exchange into temp + reduce_add twice) */
+    SAR_OP_REDUCE_INTO = 2, /* dst += src                                   (recv into temp + reduce_add)           */
+    SAR_OP_MREDUCE = 3      /* dst(s) <- ring-ordered sum over a rank group (the NCCL pre-work collectives)         */
+};
+
+#define SAR_MAX_RANKS 64
+
+typedef struct sar_ctx sar_ctx;
+typedef struct sar_schedule sar_schedule;
+
+/* one lowered schedule row, as reported by sar_schedule_op() */
+typedef struct sar_op_info {
+    int32_t kind;        /* SAR_OP_*                                                        */
+    int32_t dst_rank;    /* COPY/REDUCE_INTO/MREDUCE: destination; XREDUCE: first side      */
+    int32_t src_rank;    /* COPY/REDUCE_INTO: source; XREDUCE: second side; MREDUCE: -1     */
+    int32_t dst_chunk;   /* first chunk written, in units of the schedule's `parts`         */
+    int32_t src_chunk;   /* first chunk read                                                */
+    int32_t nchunks;     /* consecutive chunks moved                                        */
+    int32_t group;       /* MREDUCE: ranks 0..group-1 take part                             */
+    int32_t bcast;       /* MREDUCE: 1 = every group member receives the result             */
+    int32_t to_end;      /* 1 = the range also takes the elements past parts*chunk          */
+} sar_op_info;
+
+typedef struct sar_stats_t {
+    uint64_t algorithmic_bytes;    /* minimum bytes the prepared main schedule must move (see sar_schedule_bytes) */
+    uint64_t reference_op_bytes;   /* bytes of the reference's own op sequence (temp staging + reduce_add)        */
+    uint64_t prework_bytes;        /* algorithmic bytes of the prepared pre-work schedule, 0 if none              */
+    int32_t rounds;                /* rounds of the main schedule                                                 */
+    int32_t launches;              /* kernel launches per sar_run (main + pre-work, sleep excluded)               */
+    int32_t ops;                   /* rows of the main schedule                                                   */
+    int32_t uses_graph;            /* 1 if sar_run replays a hipGraph                                             */
+} sar_stats_t;
+
+/* run-time tunables of the round kernel; sar_get_tuning() reports the defaults */
+typedef struct sar_tuning_t {
+    int32_t block;        /* threads per workgroup: 256 or 512                                       */
+    int32_t unroll;       /* 16-byte vectors per thread and stream: 1, 2, 4 or 8                     */
+    int32_t order;        /* 0 = tiles op by op, 1 = tiles of a round's ops interleaved              */
+    int32_t cache_policy; /* 0 = all accesses cached, 1 = all streaming (nontemporal), 2 = planned:  */
+                          /*     streaming unless the data is read again within `reuse_rounds`       */
+    int32_t reuse_rounds; /* look-ahead of policy 2, in rounds                                       */
+    int32_t reverse_odd;  /* 1 = odd rounds walk their tiles backwards (keeps the cache tail warm)   */
+} sar_tuning_t;
+
+/* ---- library ------------------------------------------------------- */
+int sar_version(void);
+const char* sar_last_error(void);
+
+/* Number of HIP devices.  Replaces cudaGetDeviceCount + "Need at least %d
+ * GPUs" (allreduce_8GPU.cu:932-937): one device is enough here. */
+int sar_device_count(int* count);
+
+/* pad_buffers.py:31-48: chunk = (bytes/(n-1)/1024 + 1)*1024, padded =
+ * chunk*(n-1).  Always grows, also when bytes is already divisible. */
+uint64_t sar_pad_bytes(uint64_t bytes, int n);
+
+/* ---- schedules (host only; usable without a GPU) -------------------- */
+
+/* Parse a table in the text format the reference synthesizers print
+ * (synthesizer_pow2.py:241-247, matching strings :54,:71,:84).  Closes the
+ * reference's manual step "translate the output into ncclSend/ncclRecv by
+ * hand" (README.md:35). */
+int sar_schedule_parse(const char* text, size_t len, int n, sar_schedule** out);
+
+/* Built-in tables.  alg is one of
+ *   "stragglar"   the table hard-coded in stragglar_allreduce_helper
+ *                 (allreduce_8GPU.cu:555-874 for n=8, allreduce_4GPU.cu:299-368 for n=4)
+ *   "ring"        ring_allreduce_helper  (allreduce_8GPU.cu:146-198), any n >= 2
+ *   "rhd"         rhd_allreduce_helper   (allreduce_8GPU.cu:221-532, allreduce_4GPU.cu:196-278), n a power of two
+ *   "direct"      direct_allreduce_helper (allreduce_8GPU.cu:60-113, allreduce_4GPU.cu:56-92), even n
+ *   "prework_rs"  the (n-1)-rank in-place ncclReduceScatter (allreduce_8GPU.cu:890-895, reducescatter.cu:103-108)
+ *   "prework_ar"  the (n-1)-rank ncclAllReduce before `direct` in delay mode (allreduce_8GPU.cu:129-134) */
+int sar_schedule_builtin(const char* alg, int n, sar_schedule** out);
+
+/* Structural checks: rank/chunk bounds; no row of a round writes a range that
+ * another row of the same round reads or writes; for StragglAR tables also the
+ * synthesizers' own rules (valid_round, synthesizer_pow2.py:86-103: one send
+ * and one receive per rank and round; senders hold what they send, :47,:58-59;
+ * termination with every rank holding every chunk, :213).  On failure the
+ * reason is copied into msg (if cap > 0) and SAR_ESCHED is returned. */
+int sar_schedule_validate(const sar_schedule* s, char* msg, size_t cap);
+
+int sar_schedule_ranks(const sar_schedule* s);
+int sar_schedule_parts(const sar_schedule* s);   /* chunks per rank buffer: n-1 (stragglar), n (ring, rhd), 1 (direct) */
+int sar_schedule_rounds(const sar_schedule* s);
+int sar_schedule_round_ops(const sar_schedule* s, int round);
+int sar_schedule_op(const sar_schedule* s, int round, int index, sar_op_info* out);
+
+/* Bytes one execution moves for `elems` elements of `elem_size` bytes per
+ * rank.  algorithmic: COPY 2NE, REDUCE_INTO 3NE, XREDUCE 4NE, MREDUCE
+ * (sources + destinations)NE.  reference_op: the reference's own sequence for
+ * the same rows (recv-to-temp 2NE + reduce_add 3NE per receiving side). */
+int sar_schedule_bytes(const sar_schedule* s, uint64_t elems, int elem_size,
+                       uint64_t* algorithmic, uint64_t* reference_op);
+
+void sar_schedule_free(sar_schedule* s);
+
+/* ---- device context -------------------------------------------------- */
+
+/* Replaces the per-process setup of main() (allreduce_8GPU.cu:939-963): one
+ * device, one stream for the ranks that are on time and one for the straggler. */
+int sar_create(int device, sar_ctx** out);
+void sar_destroy(sar_ctx* ctx);
+
+/* Rank buffers, replacing cudaMallocAsync(d_buffers[i]) (allreduce_8GPU.cu
+ * :977-990).  No temp buffers exist: exchanges are fused.  All ranks share one
+ * arena; rank r starts at r*stride, stride = bytes rounded up to 2 MiB. */
+int sar_alloc_ranks(sar_ctx* ctx, int n, uint64_t bytes_per_rank, int dtype);
+
+int sar_upload(sar_ctx* ctx, int rank, uint64_t byte_off, const void* host, uint64_t bytes);
+int sar_download(sar_ctx* ctx, int rank, uint64_t byte_off, void* host, uint64_t bytes);
+
+/* fill_pattern (allreduce_8GPU.cu:41-45) on elements [elem_off, elem_off+elems) of one rank. */
+int sar_fill_const(sar_ctx* ctx, int rank, uint64_t elem_off, uint64_t elems, double value);
+
+/* The reference's per-iteration self-check fill (allreduce_8GPU.cu:1011-1021,
+ * allreduce_4GPU.cu:535-545): rank i <- i+base; with delay < 0 `direct`
+ * pre-fills ranks < n-1, and `stragglar` chunk i of rank i < n-1, with the sum
+ * of the first n-1 constants. */
+int sar_fill_reference_pattern(sar_ctx* ctx, const char* alg, float delay_ms, int base);
+
+/* Seeded synthetic inputs generated on the device, counter-based so that the
+ * value of (seed, rank, element) does not depend on launch shape.
+ * uniform: lo + (hi-lo)*k/2^24 with k the top 24 bits of a 64-bit mix.
+ * normal:  mean + std*(sum of 12 such uniforms - 6)  (Irwin-Hall). */
+int sar_fill_uniform(sar_ctx* ctx, int rank, uint64_t seed, double lo, double hi);
+int sar_fill_normal(sar_ctx* ctx, int rank, uint64_t seed, double mean, double std);
+
+/* Keep / bring back a device-side copy of all rank buffers (the reference
+ * re-fills before every iteration, allreduce_8GPU.cu:1009-1026). */
+int sar_snapshot(sar_ctx* ctx);
+int sar_restore(sar_ctx* ctx);
+
+/* 1 if every rank buffer holds the same bits over its first parts*chunk elements. */
+int sar_ranks_identical(sar_ctx* ctx, uint64_t elems, int* identical);
+
+int sar_get_tuning(sar_ctx* ctx, sar_tuning_t* out);
+int sar_set_tuning(sar_ctx* ctx, const sar_tuning_t* in);   /* takes effect at the next sar_prepare */
+
+/* Lower `main` (and the optional pre-work run before it in delay mode) onto
+ * the allocated ranks: per-round op tables in device memory, launch shapes,
+ * and with use_graph != 0 a captured hipGraph of the main rounds.  Replaces
+ * the unrolled bodies of the *_allreduce_helper functions. */
+int sar_prepare(sar_ctx* ctx, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph);
+
+/* One timed execution = one call of stragglar_allreduce / ring_allreduce /
+ * ... (delay < 0, allreduce_8GPU.cu:900-905) or of their *_delay variants
+ * (delay >= 0, :876-898): start event, the straggler's stream sleeps
+ * delay_ms while the pre-work runs, then the rounds, stop event, block on
+ * stop.  elapsed_ms is stop - start as in the reference (:1052). */
+int sar_run(sar_ctx* ctx, float delay_ms, float* elapsed_ms);
+
+/* Same as sar_run with delay < 0 and no graph, with an event pair around
+ * every launch: ms[i] is the duration of launch i (at most cap written,
+ * *count = launches). */
+int sar_run_profiled(sar_ctx* ctx, float* ms, int cap, int* count);
+
+/* Algorithmic bytes of each launch of the prepared main schedule, in launch
+ * order (the denominator-free half of a per-kernel roofline figure). */
+int sar_launch_bytes(sar_ctx* ctx, uint64_t* bytes, int cap, int* count);
+
+/* Ticks of the device's constant-rate wall clock that delay_ms lasts: the
+ * figure the CLI prints as "Sleep cycles" (calculate_sleep_cycles,
+ * allreduce_8GPU.cu:47-58, uses ms * clockRate_kHz of the shader clock). */
+int sar_sleep_ticks(sar_ctx* ctx, float delay_ms, int64_t* ticks);
+
+int sar_stats(sar_ctx* ctx, sar_stats_t* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAR_H */

@@ -1,0 +1,327 @@
+"""ctypes binding of the C ABI declared in ``include/sar.h``.
+
+The shared library is built in-tree by ``stragglar_amd/csrc/Makefile``.  There
+is no fallback: if the library is missing or no HIP device is usable, the
+calls raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libsar_hip.so")
+
+DTYPES = {"f32": 0, "f16": 1, "bf16": 2}
+ELEM_SIZE = {"f32": 4, "f16": 2, "bf16": 2}
+OP_KINDS = {0: "copy", 1: "xreduce", 2: "reduce_into", 3: "mreduce"}
+
+
+class SarError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__("sar error %d: %s" % (code, message))
+        self.code = code
+        self.message = message
+
+
+class OpInfo(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in
+                ("kind", "dst_rank", "src_rank", "dst_chunk", "src_chunk", "nchunks", "group", "bcast", "to_end")]
+
+    def as_tuple(self):
+        return tuple(getattr(self, n) for n, _ in self._fields_)
+
+
+class Stats(ctypes.Structure):
+    _fields_ = [("algorithmic_bytes", ctypes.c_uint64), ("reference_op_bytes", ctypes.c_uint64),
+                ("prework_bytes", ctypes.c_uint64), ("rounds", ctypes.c_int32), ("launches", ctypes.c_int32),
+                ("ops", ctypes.c_int32), ("uses_graph", ctypes.c_int32)]
+
+
+class Tuning(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd")]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def build_library() -> str:
+    """Compile the HIP library and the CLI drivers for gfx950 (hipcc, in-tree)."""
+    subprocess.run(["make", "-C", os.path.join(_HERE, "csrc"), "-j4", "-s"], check=True)
+    return _LIB_PATH
+
+
+EXPORTS = [
+    "sar_version", "sar_last_error", "sar_device_count", "sar_pad_bytes",
+    "sar_schedule_parse", "sar_schedule_builtin", "sar_schedule_validate", "sar_schedule_ranks",
+    "sar_schedule_parts", "sar_schedule_rounds", "sar_schedule_round_ops", "sar_schedule_op",
+    "sar_schedule_bytes", "sar_schedule_free",
+    "sar_create", "sar_destroy", "sar_alloc_ranks", "sar_upload", "sar_download", "sar_fill_const",
+    "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
+    "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
+    "sar_launch_bytes", "sar_sleep_ticks", "sar_stats",
+]
+
+
+class Library:
+    """The loaded shared object with argument types declared."""
+
+    def __init__(self, path: Optional[str] = None):
+        path = path or _LIB_PATH
+        if not os.path.exists(path):
+            raise FileNotFoundError(
+                "%s is missing: build it with `make -C stragglar_amd/csrc` (there is no CPU fallback)" % path)
+        self.path = path
+        L = self.lib = ctypes.CDLL(path)
+        vp, c_int, u64, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_size_t
+        P = ctypes.POINTER
+        sig = {
+            "sar_version": (c_int, []),
+            "sar_last_error": (ctypes.c_char_p, []),
+            "sar_device_count": (c_int, [P(c_int)]),
+            "sar_pad_bytes": (u64, [u64, c_int]),
+            "sar_schedule_parse": (c_int, [ctypes.c_char_p, sz, c_int, P(vp)]),
+            "sar_schedule_builtin": (c_int, [ctypes.c_char_p, c_int, P(vp)]),
+            "sar_schedule_validate": (c_int, [vp, ctypes.c_char_p, sz]),
+            "sar_schedule_ranks": (c_int, [vp]),
+            "sar_schedule_parts": (c_int, [vp]),
+            "sar_schedule_rounds": (c_int, [vp]),
+            "sar_schedule_round_ops": (c_int, [vp, c_int]),
+            "sar_schedule_op": (c_int, [vp, c_int, c_int, P(OpInfo)]),
+            "sar_schedule_bytes": (c_int, [vp, u64, c_int, P(u64), P(u64)]),
+            "sar_schedule_free": (None, [vp]),
+            "sar_create": (c_int, [c_int, P(vp)]),
+            "sar_destroy": (None, [vp]),
+            "sar_alloc_ranks": (c_int, [vp, c_int, u64, c_int]),
+            "sar_upload": (c_int, [vp, c_int, u64, vp, u64]),
+            "sar_download": (c_int, [vp, c_int, u64, vp, u64]),
+            "sar_fill_const": (c_int, [vp, c_int, u64, u64, ctypes.c_double]),
+            "sar_fill_reference_pattern": (c_int, [vp, ctypes.c_char_p, ctypes.c_float, c_int]),
+            "sar_fill_uniform": (c_int, [vp, c_int, u64, ctypes.c_double, ctypes.c_double]),
+            "sar_fill_normal": (c_int, [vp, c_int, u64, ctypes.c_double, ctypes.c_double]),
+            "sar_snapshot": (c_int, [vp]),
+            "sar_restore": (c_int, [vp]),
+            "sar_ranks_identical": (c_int, [vp, u64, P(c_int)]),
+            "sar_get_tuning": (c_int, [vp, P(Tuning)]),
+            "sar_set_tuning": (c_int, [vp, P(Tuning)]),
+            "sar_prepare": (c_int, [vp, vp, vp, c_int]),
+            "sar_run": (c_int, [vp, ctypes.c_float, P(ctypes.c_float)]),
+            "sar_run_profiled": (c_int, [vp, P(ctypes.c_float), c_int, P(c_int)]),
+            "sar_launch_bytes": (c_int, [vp, P(u64), c_int, P(c_int)]),
+            "sar_sleep_ticks": (c_int, [vp, ctypes.c_float, P(ctypes.c_int64)]),
+            "sar_stats": (c_int, [vp, P(Stats)]),
+        }
+        assert sorted(sig) == sorted(EXPORTS)
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+
+    def check(self, rc: int):
+        if rc != 0:
+            raise SarError(rc, (self.lib.sar_last_error() or b"").decode())
+
+    def device_count(self) -> int:
+        n = ctypes.c_int(0)
+        self.check(self.lib.sar_device_count(ctypes.byref(n)))
+        return n.value
+
+    def pad_bytes(self, nbytes: int, n: int) -> int:
+        return int(self.lib.sar_pad_bytes(nbytes, n))
+
+    def parse(self, text: str, n: int) -> "Schedule":
+        raw = text.encode()
+        h = ctypes.c_void_p()
+        self.check(self.lib.sar_schedule_parse(raw, len(raw), n, ctypes.byref(h)))
+        return Schedule(self, h)
+
+    def builtin(self, alg: str, n: int) -> "Schedule":
+        h = ctypes.c_void_p()
+        self.check(self.lib.sar_schedule_builtin(alg.encode(), n, ctypes.byref(h)))
+        return Schedule(self, h)
+
+    def context(self, device: int = 0) -> "Context":
+        h = ctypes.c_void_p()
+        self.check(self.lib.sar_create(device, ctypes.byref(h)))
+        return Context(self, h)
+
+
+_default: Optional[Library] = None
+
+
+def load_library() -> Library:
+    global _default
+    if _default is None:
+        _default = Library()
+    return _default
+
+
+class Schedule:
+    def __init__(self, lib: Library, handle):
+        self._lib, self._h = lib, handle
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.lib.sar_schedule_free(self._h)
+            self._h = None
+
+    @property
+    def handle(self):
+        return self._h
+
+    @property
+    def ranks(self) -> int:
+        return self._lib.lib.sar_schedule_ranks(self._h)
+
+    @property
+    def parts(self) -> int:
+        return self._lib.lib.sar_schedule_parts(self._h)
+
+    @property
+    def num_rounds(self) -> int:
+        return self._lib.lib.sar_schedule_rounds(self._h)
+
+    def validate(self) -> str:
+        """'' if valid, else the reason."""
+        buf = ctypes.create_string_buffer(512)
+        rc = self._lib.lib.sar_schedule_validate(self._h, buf, len(buf))
+        return "" if rc == 0 else (buf.value.decode() or "invalid")
+
+    def rounds(self) -> List[List[tuple]]:
+        """Rows as (kind, dst_rank, src_rank, dst_chunk, src_chunk, nchunks, group, bcast, to_end)."""
+        out = []
+        for r in range(self.num_rounds):
+            k = self._lib.lib.sar_schedule_round_ops(self._h, r)
+            row = []
+            for i in range(k):
+                info = OpInfo()
+                self._lib.check(self._lib.lib.sar_schedule_op(self._h, r, i, ctypes.byref(info)))
+                row.append(info.as_tuple())
+            out.append(row)
+        return out
+
+    def bytes(self, elems: int, elem_size: int):
+        a, b = ctypes.c_uint64(0), ctypes.c_uint64(0)
+        self._lib.check(self._lib.lib.sar_schedule_bytes(self._h, elems, elem_size, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
+
+
+class Context:
+    def __init__(self, lib: Library, handle):
+        self._lib, self._h = lib, handle
+        self.n = 0
+        self.dtype = "f32"
+        self.bytes_per_rank = 0
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.lib.sar_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def _c(self, rc):
+        self._lib.check(rc)
+
+    def alloc_ranks(self, n: int, bytes_per_rank: int, dtype: str = "f32"):
+        self._c(self._lib.lib.sar_alloc_ranks(self._h, n, bytes_per_rank, DTYPES[dtype]))
+        self.n, self.dtype, self.bytes_per_rank = n, dtype, bytes_per_rank
+
+    @property
+    def elems(self) -> int:
+        return self.bytes_per_rank // ELEM_SIZE[self.dtype]
+
+    def upload(self, rank: int, arr: np.ndarray, byte_off: int = 0):
+        arr = np.ascontiguousarray(arr)
+        self._c(self._lib.lib.sar_upload(self._h, rank, byte_off, arr.ctypes.data, arr.nbytes))
+
+    def download(self, rank: int, byte_off: int = 0, nbytes: Optional[int] = None) -> np.ndarray:
+        nbytes = self.bytes_per_rank - byte_off if nbytes is None else nbytes
+        np_dt = np.float32 if self.dtype == "f32" else np.uint16
+        out = np.empty(nbytes // np.dtype(np_dt).itemsize, dtype=np_dt)
+        self._c(self._lib.lib.sar_download(self._h, rank, byte_off, out.ctypes.data, out.nbytes))
+        return out
+
+    def fill_const(self, rank: int, value: float, elem_off: int = 0, elems: Optional[int] = None):
+        elems = self.elems - elem_off if elems is None else elems
+        self._c(self._lib.lib.sar_fill_const(self._h, rank, elem_off, elems, float(value)))
+
+    def fill_reference_pattern(self, alg: str, delay_ms: float, base: int):
+        self._c(self._lib.lib.sar_fill_reference_pattern(self._h, alg.encode(), float(delay_ms), base))
+
+    def fill_uniform(self, rank: int, seed: int, lo: float, hi: float):
+        self._c(self._lib.lib.sar_fill_uniform(self._h, rank, seed, lo, hi))
+
+    def fill_normal(self, rank: int, seed: int, mean: float, std: float):
+        self._c(self._lib.lib.sar_fill_normal(self._h, rank, seed, mean, std))
+
+    def snapshot(self):
+        self._c(self._lib.lib.sar_snapshot(self._h))
+
+    def restore(self):
+        self._c(self._lib.lib.sar_restore(self._h))
+
+    def ranks_identical(self, elems: Optional[int] = None) -> bool:
+        flag = ctypes.c_int(0)
+        self._c(self._lib.lib.sar_ranks_identical(self._h, self.elems if elems is None else elems, ctypes.byref(flag)))
+        return bool(flag.value)
+
+    def get_tuning(self) -> Tuning:
+        t = Tuning()
+        self._c(self._lib.lib.sar_get_tuning(self._h, ctypes.byref(t)))
+        return t
+
+    def set_tuning(self, **kw):
+        t = self.get_tuning()
+        for k, v in kw.items():
+            if not hasattr(t, k):
+                raise KeyError(k)
+            setattr(t, k, v)
+        self._c(self._lib.lib.sar_set_tuning(self._h, ctypes.byref(t)))
+
+    def prepare(self, main: Schedule, prework: Optional[Schedule] = None, use_graph: bool = False):
+        self._c(self._lib.lib.sar_prepare(self._h, prework.handle if prework else None, main.handle, int(use_graph)))
+
+    def run(self, delay_ms: float = -1.0) -> float:
+        ms = ctypes.c_float(0)
+        self._c(self._lib.lib.sar_run(self._h, float(delay_ms), ctypes.byref(ms)))
+        return ms.value
+
+    def run_profiled(self) -> List[float]:
+        cap = 4096
+        buf = (ctypes.c_float * cap)()
+        cnt = ctypes.c_int(0)
+        self._c(self._lib.lib.sar_run_profiled(self._h, buf, cap, ctypes.byref(cnt)))
+        return [buf[i] for i in range(min(cap, cnt.value))]
+
+    def launch_bytes(self) -> List[int]:
+        cap = 4096
+        buf = (ctypes.c_uint64 * cap)()
+        cnt = ctypes.c_int(0)
+        self._c(self._lib.lib.sar_launch_bytes(self._h, buf, cap, ctypes.byref(cnt)))
+        return [int(buf[i]) for i in range(min(cap, cnt.value))]
+
+    def sleep_ticks(self, delay_ms: float) -> int:
+        t = ctypes.c_int64(0)
+        self._c(self._lib.lib.sar_sleep_ticks(self._h, float(delay_ms), ctypes.byref(t)))
+        return t.value
+
+    def stats(self) -> Stats:
+        s = Stats()
+        self._c(self._lib.lib.sar_stats(self._h, ctypes.byref(s)))
+        return s

@@ -1,0 +1,623 @@
+// Host executor and C ABI: rank arena in HBM, lowering of a schedule to
+// per-round op tables, cache-policy planning, launch / hipGraph replay, timing.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "kernels.hpp"
+#include "sar.h"
+#include "schedule.hpp"
+
+namespace {
+
+thread_local std::string g_error;
+
+int set_error(int code, const std::string& msg) { g_error = msg; return code; }
+
+#define SAR_HIP(expr)                                                                                   \
+    do {                                                                                                \
+        hipError_t e_ = (expr);                                                                         \
+        if (e_ != hipSuccess)                                                                           \
+            return set_error(SAR_EHIP, std::string(#expr) + ": " + hipGetErrorString(e_));              \
+    } while (0)
+
+constexpr uint64_t kArenaAlign = 2ull << 20;   // rank bases on 2 MiB boundaries (one large-page fragment each)
+constexpr float kMaxDelayMs = 60000.f;
+
+// One kernel launch: the rows of a round that share a kernel (COPY /
+// REDUCE_INTO / XREDUCE in one, MREDUCE in the other).
+struct Launch {
+    uint32_t first_op = 0, nops = 0, total_tiles = 0, tiles_per_op = 0, reverse = 0;
+    bool mreduce = false;
+    uint64_t algorithmic_bytes = 0;
+};
+
+int elem_size_of(int dtype) { return dtype == SAR_F32 ? 4 : 2; }
+
+}  // namespace
+
+struct sar_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr, straggler_stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr, ev_join = nullptr;
+    std::vector<hipEvent_t> ev_prof;
+    int wall_khz = 100000;
+
+    int n = 0, dtype = SAR_F32;
+    uint64_t bytes_per_rank = 0, stride = 0;
+    char* arena = nullptr;
+    char* snapshot = nullptr;
+    int* d_flag = nullptr;
+
+    sar_tuning_t tune{256, 2, 0, 2, 1, 1};
+
+    // prepared plan
+    bool prepared = false;
+    sar::DevOp* d_ops = nullptr;
+    char** d_ptrs = nullptr;
+    std::vector<Launch> prework, rounds;
+    sar_stats_t stats{};
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+
+    char* rank_base(int r) const { return arena + (uint64_t)r * stride; }
+    uint64_t elems() const { return bytes_per_rank / (uint64_t)elem_size_of(dtype); }
+};
+
+namespace {
+
+void drop_plan(sar_ctx* c) {
+    if (c->graph_exec) { (void)hipGraphExecDestroy(c->graph_exec); c->graph_exec = nullptr; }
+    if (c->graph) { (void)hipGraphDestroy(c->graph); c->graph = nullptr; }
+    if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
+    if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
+    c->prework.clear(); c->rounds.clear(); c->prepared = false;
+    c->stats = sar_stats_t{};
+}
+
+void drop_ranks(sar_ctx* c) {
+    drop_plan(c);
+    if (c->arena) { (void)hipFree(c->arena); c->arena = nullptr; }
+    if (c->snapshot) { (void)hipFree(c->snapshot); c->snapshot = nullptr; }
+    c->n = 0; c->bytes_per_rank = 0; c->stride = 0;
+}
+
+// A byte interval of one rank buffer that a row reads or writes.
+struct Touch { int rank; uint64_t lo, hi; };
+
+struct RowAccess {
+    std::vector<Touch> reads, writes;   // writes[0] belongs to p0, writes[1] to p1 (XREDUCE)
+};
+
+bool overlaps(const Touch& a, const Touch& b) { return a.rank == b.rank && a.lo < b.hi && b.lo < a.hi; }
+
+RowAccess accesses(const sar::Schedule& s, const sar::Op& op, uint64_t elems, int es) {
+    sar::Range r = sar::lower_range(s, op, elems);
+    RowAccess a;
+    uint64_t dlo = r.dst_off * es, slo = r.src_off * es, len = r.len * es;
+    switch (op.kind) {
+        case SAR_OP_COPY:
+            a.reads.push_back({op.src_rank, slo, slo + len});
+            a.writes.push_back({op.dst_rank, dlo, dlo + len});
+            break;
+        case SAR_OP_REDUCE_INTO:
+            a.reads.push_back({op.dst_rank, dlo, dlo + len});
+            a.reads.push_back({op.src_rank, slo, slo + len});
+            a.writes.push_back({op.dst_rank, dlo, dlo + len});
+            break;
+        case SAR_OP_XREDUCE:
+            a.reads.push_back({op.dst_rank, dlo, dlo + len});
+            a.reads.push_back({op.src_rank, slo, slo + len});
+            a.writes.push_back({op.dst_rank, dlo, dlo + len});
+            a.writes.push_back({op.src_rank, slo, slo + len});
+            break;
+        default:
+            for (int q = 0; q < op.group; ++q) a.reads.push_back({q, dlo, dlo + len});
+            if (op.bcast) { for (int q = 0; q < op.group; ++q) a.writes.push_back({q, dlo, dlo + len}); }
+            else a.writes.push_back({op.dst_rank, dlo, dlo + len});
+            break;
+    }
+    return a;
+}
+
+// Lower every round of `s` to device rows appended to `rows` / `ptrs`.
+int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std::vector<char*>& ptrs, std::vector<Launch>& out,
+          const sar::Schedule* next /* schedule that runs afterwards, for the cache look-ahead */) {
+    const int es = elem_size_of(c->dtype);
+    const uint64_t elems = c->elems();
+    const uint64_t round_tile_bytes = (uint64_t)c->tune.block * (uint64_t)c->tune.unroll * 16u;
+
+    // per-round access lists, including those of the schedule that follows
+    std::vector<std::vector<RowAccess>> acc;
+    for (const auto& round : s.rounds) {
+        std::vector<RowAccess> v;
+        for (const auto& op : round) v.push_back(accesses(s, op, elems, es));
+        acc.push_back(v);
+    }
+    const size_t own_rounds = acc.size();
+    if (next)
+        for (const auto& round : next->rounds) {
+            std::vector<RowAccess> v;
+            for (const auto& op : round) v.push_back(accesses(*next, op, elems, es));
+            acc.push_back(v);
+        }
+    auto read_soon = [&](size_t round, const Touch& t) {
+        size_t last = std::min(acc.size(), round + 1 + (size_t)std::max(0, c->tune.reuse_rounds));
+        for (size_t r = round + 1; r < last; ++r)
+            for (const auto& ra : acc[r])
+                for (const auto& rd : ra.reads)
+                    if (overlaps(rd, t)) return true;
+        return false;
+    };
+
+    for (size_t ri = 0; ri < own_rounds; ++ri) {
+      const auto& round = s.rounds[ri];
+      for (int cls = 0; cls < 2; ++cls) {
+        const uint64_t tile_bytes = cls ? sar::mreduce_tile_bytes() : round_tile_bytes;
+        Launch L; L.first_op = (uint32_t)rows.size(); L.mreduce = cls != 0;
+        uint64_t tiles = 0; bool uniform = true; uint64_t first_tiles = 0;
+        for (size_t oi = 0; oi < round.size(); ++oi) {
+            const sar::Op& op = round[oi];
+            if ((op.kind == SAR_OP_MREDUCE) != (cls != 0)) continue;
+            sar::Range rg = sar::lower_range(s, op, elems);
+            uint64_t bytes = rg.len * es;
+            if (bytes == 0) continue;   // buffer shorter than `parts` elements: nothing to move
+            uint64_t doff = rg.dst_off * es, soff = rg.src_off * es;
+            if (doff + bytes > c->bytes_per_rank || soff + bytes > c->bytes_per_rank) return set_error(SAR_ESCHED, "row leaves the rank buffer");
+            sar::DevOp d{};
+            d.kind = (uint32_t)op.kind; d.bytes = bytes;
+            bool aligned = true;
+            if (op.kind == SAR_OP_MREDUCE) {
+                // ring order over the group: x_{r+1}, x_{r+2}, ..., x_{r-1}, x_r (the owner last)
+                d.ptr_off = (uint32_t)ptrs.size(); d.nsrc = (uint32_t)op.group;
+                for (int j = 1; j <= op.group; ++j) ptrs.push_back(c->rank_base((op.dst_rank + j) % op.group) + doff);
+                if (op.bcast) { d.ndst = (uint32_t)op.group; for (int q = 0; q < op.group; ++q) ptrs.push_back(c->rank_base(q) + doff); }
+                else { d.ndst = 1; ptrs.push_back(c->rank_base(op.dst_rank) + doff); }
+                for (size_t k = d.ptr_off; k < ptrs.size(); ++k) aligned &= ((uintptr_t)ptrs[k] & 15u) == 0;
+            } else {
+                d.p0 = c->rank_base(op.dst_rank) + doff;
+                d.p1 = c->rank_base(op.src_rank) + soff;
+                aligned = (((uintptr_t)d.p0 | (uintptr_t)d.p1) & 15u) == 0;
+            }
+            if (aligned) d.flags |= sar::DEVOP_VEC;
+            // cache policy
+            const RowAccess& ra = acc[ri][oi];
+            if (c->tune.cache_policy == 1) {
+                d.flags |= sar::DEVOP_LNT | sar::DEVOP_SNT0 | sar::DEVOP_SNT1;
+            } else if (c->tune.cache_policy == 2) {
+                bool any_read_again = false;
+                for (const auto& rd : ra.reads) any_read_again |= read_soon(ri, rd);
+                if (!any_read_again) d.flags |= sar::DEVOP_LNT;
+                if (op.kind == SAR_OP_MREDUCE) {
+                    bool again = false;
+                    for (const auto& w : ra.writes) again |= read_soon(ri, w);
+                    if (!again) d.flags |= sar::DEVOP_SNT0;
+                } else {
+                    if (!read_soon(ri, ra.writes[0])) d.flags |= sar::DEVOP_SNT0;
+                    if (ra.writes.size() > 1 && !read_soon(ri, ra.writes[1])) d.flags |= sar::DEVOP_SNT1;
+                }
+            }
+            uint64_t nt = (bytes + tile_bytes - 1) / tile_bytes;
+            if (tiles + nt > 0x7fffffffull) return set_error(SAR_EINVAL, "round needs more than 2^31 tiles");
+            d.tile_begin = (uint32_t)tiles; d.ntiles = (uint32_t)nt;
+            if (L.nops == 0) first_tiles = nt; else uniform &= (nt == first_tiles);
+            tiles += nt;
+            uint64_t k = 0;
+            switch (op.kind) {
+                case SAR_OP_COPY: k = 2; break;
+                case SAR_OP_REDUCE_INTO: k = 3; break;
+                case SAR_OP_XREDUCE: k = 4; break;
+                default: k = d.nsrc + d.ndst; break;
+            }
+            L.algorithmic_bytes += k * bytes;
+            rows.push_back(d); L.nops++;
+        }
+        if (L.nops == 0) continue;
+        L.total_tiles = (uint32_t)tiles;
+        L.tiles_per_op = uniform ? (uint32_t)first_tiles : 0;
+        L.reverse = (c->tune.reverse_odd && (ri & 1)) ? 1u : 0u;
+        out.push_back(L);
+      }
+    }
+    return SAR_OK;
+}
+
+int launch_one(sar_ctx* c, const Launch& L) {
+    if (L.total_tiles == 0) return SAR_OK;
+    const uint32_t interleave = (uint32_t)(c->tune.order == 1);
+    if (L.mreduce)
+        SAR_HIP(sar::launch_mreduce(c->dtype, c->stream, c->d_ops + L.first_op, L.nops, c->d_ptrs, L.total_tiles, L.tiles_per_op, interleave, L.reverse));
+    else
+        SAR_HIP(sar::launch_round(c->dtype, c->tune.unroll, c->tune.block, c->stream, c->d_ops + L.first_op, L.nops,
+                                  L.total_tiles, L.tiles_per_op, interleave, L.reverse));
+    return SAR_OK;
+}
+
+int launch_all(sar_ctx* c, const std::vector<Launch>& v) {
+    for (const auto& L : v) { int rc = launch_one(c, L); if (rc) return rc; }
+    return SAR_OK;
+}
+
+bool valid_tuning(const sar_tuning_t& t) {
+    return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
+           (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
+           (t.reverse_odd == 0 || t.reverse_odd == 1);
+}
+
+}  // namespace
+
+extern "C" {
+
+int sar_version(void) { return SAR_VERSION; }
+const char* sar_last_error(void) { return g_error.c_str(); }
+
+int sar_device_count(int* count) {
+    if (!count) return set_error(SAR_EINVAL, "count is null");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) { *count = 0; (void)hipGetLastError(); return set_error(SAR_ENODEV, std::string("hipGetDeviceCount: ") + hipGetErrorString(e)); }
+    *count = n;
+    return SAR_OK;
+}
+
+uint64_t sar_pad_bytes(uint64_t bytes, int n) { return sar::pad_bytes(bytes, n); }
+
+// ---- schedules ---------------------------------------------------------------
+
+int sar_schedule_parse(const char* text, size_t len, int n, sar_schedule** out) {
+    if (!out) return set_error(SAR_EINVAL, "out is null");
+    *out = nullptr;
+    try {
+        sar_schedule* s = new sar_schedule{sar::parse_table(text, len, n)};
+        *out = s; return SAR_OK;
+    } catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory");
+    } catch (const std::exception& e) { return set_error(SAR_EPARSE, e.what()); }
+}
+
+int sar_schedule_builtin(const char* alg, int n, sar_schedule** out) {
+    if (!out || !alg) return set_error(SAR_EINVAL, "null argument");
+    *out = nullptr;
+    try {
+        sar_schedule* s = new sar_schedule{sar::builtin(alg, n)};
+        *out = s; return SAR_OK;
+    } catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory");
+    } catch (const std::exception& e) { return set_error(SAR_EINVAL, e.what()); }
+}
+
+int sar_schedule_validate(const sar_schedule* s, char* msg, size_t cap) {
+    if (!s) return set_error(SAR_EINVAL, "schedule is null");
+    std::string why;
+    try { why = sar::validate(s->s); } catch (const std::exception& e) { why = e.what(); }
+    if (msg && cap) { std::snprintf(msg, cap, "%s", why.c_str()); }
+    if (!why.empty()) return set_error(SAR_ESCHED, why);
+    return SAR_OK;
+}
+
+int sar_schedule_ranks(const sar_schedule* s) { return s ? s->s.n : SAR_EINVAL; }
+int sar_schedule_parts(const sar_schedule* s) { return s ? s->s.parts : SAR_EINVAL; }
+int sar_schedule_rounds(const sar_schedule* s) { return s ? (int)s->s.rounds.size() : SAR_EINVAL; }
+int sar_schedule_round_ops(const sar_schedule* s, int round) {
+    if (!s || round < 0 || round >= (int)s->s.rounds.size()) return set_error(SAR_EINVAL, "round out of range");
+    return (int)s->s.rounds[round].size();
+}
+int sar_schedule_op(const sar_schedule* s, int round, int index, sar_op_info* out) {
+    if (!s || !out || round < 0 || round >= (int)s->s.rounds.size()) return set_error(SAR_EINVAL, "round out of range");
+    const auto& r = s->s.rounds[round];
+    if (index < 0 || index >= (int)r.size()) return set_error(SAR_EINVAL, "row out of range");
+    const sar::Op& o = r[index];
+    out->kind = o.kind; out->dst_rank = o.dst_rank; out->src_rank = o.src_rank; out->dst_chunk = o.dst_chunk;
+    out->src_chunk = o.src_chunk; out->nchunks = o.nchunks; out->group = o.group; out->bcast = o.bcast; out->to_end = o.to_end;
+    return SAR_OK;
+}
+
+int sar_schedule_bytes(const sar_schedule* s, uint64_t elems, int elem_size, uint64_t* algorithmic, uint64_t* reference_op) {
+    if (!s || elem_size < 1) return set_error(SAR_EINVAL, "bad argument");
+    sar::byte_counts(s->s, elems, elem_size, algorithmic, reference_op);
+    return SAR_OK;
+}
+
+void sar_schedule_free(sar_schedule* s) { delete s; }
+
+// ---- context -------------------------------------------------------------------
+
+int sar_create(int device, sar_ctx** out) {
+    if (!out) return set_error(SAR_EINVAL, "out is null");
+    *out = nullptr;
+    int count = 0;
+    int rc = sar_device_count(&count);
+    if (rc) return rc;
+    if (count < 1) return set_error(SAR_ENODEV, "no HIP device: this library has no CPU path");
+    if (device < 0 || device >= count) return set_error(SAR_EINVAL, "device index out of range");
+    SAR_HIP(hipSetDevice(device));
+    sar_ctx* c = new (std::nothrow) sar_ctx();
+    if (!c) return set_error(SAR_ENOMEM, "out of host memory");
+    c->device = device;
+    hipError_t e;
+    if ((e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess ||
+        (e = hipStreamCreateWithFlags(&c->straggler_stream, hipStreamNonBlocking)) != hipSuccess ||
+        (e = hipEventCreate(&c->ev_start)) != hipSuccess || (e = hipEventCreate(&c->ev_stop)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&c->ev_join, hipEventDisableTiming)) != hipSuccess ||
+        (e = hipMalloc((void**)&c->d_flag, sizeof(int))) != hipSuccess) {
+        sar_destroy(c);
+        return set_error(SAR_EHIP, std::string("context setup: ") + hipGetErrorString(e));
+    }
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0) c->wall_khz = khz;
+    *out = c;
+    return SAR_OK;
+}
+
+void sar_destroy(sar_ctx* c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    if (c->straggler_stream) (void)hipStreamSynchronize(c->straggler_stream);
+    drop_ranks(c);
+    for (auto e : c->ev_prof) (void)hipEventDestroy(e);
+    if (c->d_flag) (void)hipFree(c->d_flag);
+    if (c->ev_start) (void)hipEventDestroy(c->ev_start);
+    if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
+    if (c->ev_join) (void)hipEventDestroy(c->ev_join);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    if (c->straggler_stream) (void)hipStreamDestroy(c->straggler_stream);
+    delete c;
+}
+
+int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
+    if (!c) return set_error(SAR_EINVAL, "context is null");
+    if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
+    if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
+    if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    drop_ranks(c);
+    uint64_t stride = (bytes_per_rank + kArenaAlign - 1) / kArenaAlign * kArenaAlign;
+    hipError_t e = hipMalloc((void**)&c->arena, stride * (uint64_t)n);
+    if (e != hipSuccess) { (void)hipGetLastError(); c->arena = nullptr; return set_error(SAR_ENOMEM, std::string("rank arena: ") + hipGetErrorString(e)); }
+    c->n = n; c->dtype = dtype; c->bytes_per_rank = bytes_per_rank; c->stride = stride;
+    return SAR_OK;
+}
+
+static int check_rank_range(sar_ctx* c, int rank, uint64_t off, uint64_t bytes) {
+    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (rank < 0 || rank >= c->n) return set_error(SAR_EINVAL, "rank out of range");
+    if (off > c->bytes_per_rank || bytes > c->bytes_per_rank - off) return set_error(SAR_EINVAL, "range leaves the rank buffer");
+    return SAR_OK;
+}
+
+int sar_upload(sar_ctx* c, int rank, uint64_t byte_off, const void* host, uint64_t bytes) {
+    int rc = check_rank_range(c, rank, byte_off, bytes); if (rc) return rc;
+    if (!host && bytes) return set_error(SAR_EINVAL, "host pointer is null");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    if (bytes) SAR_HIP(hipMemcpy(c->rank_base(rank) + byte_off, host, bytes, hipMemcpyHostToDevice));
+    return SAR_OK;
+}
+
+int sar_download(sar_ctx* c, int rank, uint64_t byte_off, void* host, uint64_t bytes) {
+    int rc = check_rank_range(c, rank, byte_off, bytes); if (rc) return rc;
+    if (!host && bytes) return set_error(SAR_EINVAL, "host pointer is null");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    if (bytes) SAR_HIP(hipMemcpy(host, c->rank_base(rank) + byte_off, bytes, hipMemcpyDeviceToHost));
+    return SAR_OK;
+}
+
+int sar_fill_const(sar_ctx* c, int rank, uint64_t elem_off, uint64_t elems, double value) {
+    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    const uint64_t es = elem_size_of(c->dtype);
+    if (elem_off > c->elems() || elems > c->elems() - elem_off) return set_error(SAR_EINVAL, "range leaves the rank buffer");
+    int rc = check_rank_range(c, rank, elem_off * es, elems * es); if (rc) return rc;
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(sar::launch_fill_const(c->stream, c->rank_base(rank) + elem_off * es, elems, (float)value, c->dtype));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    return SAR_OK;
+}
+
+int sar_fill_reference_pattern(sar_ctx* c, const char* alg, float delay_ms, int base) {
+    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!alg) return set_error(SAR_EINVAL, "alg is null");
+    const std::string a(alg);
+    if (a != "stragglar" && a != "ring" && a != "rhd" && a != "direct") return set_error(SAR_EINVAL, "unknown algorithm");
+    const int n = c->n; const uint64_t elems = c->elems(), es = elem_size_of(c->dtype);
+    float presum = 0.f;
+    for (int i = 0; i < n - 1; ++i) presum += (float)(i + base);
+    const uint64_t chunk = elems / (uint64_t)(n - 1);
+    SAR_HIP(hipSetDevice(c->device));
+    for (int i = 0; i < n; ++i) {
+        float v = (delay_ms < 0 && a == "direct" && i < n - 1) ? presum : (float)(i + base);
+        SAR_HIP(sar::launch_fill_const(c->stream, c->rank_base(i), elems, v, c->dtype));
+        if (delay_ms < 0 && a == "stragglar" && i < n - 1)
+            SAR_HIP(sar::launch_fill_const(c->stream, c->rank_base(i) + (uint64_t)i * chunk * es, chunk, presum, c->dtype));
+    }
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    return SAR_OK;
+}
+
+static int fill_random(sar_ctx* c, int rank, uint64_t seed, double a, double b, int mode) {
+    int rc = check_rank_range(c, rank, 0, 0); if (rc) return rc;
+    SAR_HIP(hipSetDevice(c->device));
+    uint64_t key = seed * 0xD1B54A32D192ED03ull + (uint64_t)(rank + 1) * 0x8CB92BA72F3D8DD7ull;
+    SAR_HIP(sar::launch_fill_random(c->stream, c->rank_base(rank), c->elems(), key, a, b, mode, c->dtype));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    return SAR_OK;
+}
+
+int sar_fill_uniform(sar_ctx* c, int rank, uint64_t seed, double lo, double hi) { return fill_random(c, rank, seed, lo, hi - lo, 0); }
+int sar_fill_normal(sar_ctx* c, int rank, uint64_t seed, double mean, double std) { return fill_random(c, rank, seed, mean, std, 1); }
+
+int sar_snapshot(sar_ctx* c) {
+    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    SAR_HIP(hipSetDevice(c->device));
+    const uint64_t total = c->stride * (uint64_t)c->n;
+    if (!c->snapshot) {
+        hipError_t e = hipMalloc((void**)&c->snapshot, total);
+        if (e != hipSuccess) { (void)hipGetLastError(); c->snapshot = nullptr; return set_error(SAR_ENOMEM, std::string("snapshot: ") + hipGetErrorString(e)); }
+    }
+    SAR_HIP(hipMemcpyAsync(c->snapshot, c->arena, total, hipMemcpyDeviceToDevice, c->stream));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    return SAR_OK;
+}
+
+int sar_restore(sar_ctx* c) {
+    if (!c || !c->arena || !c->snapshot) return set_error(SAR_ESTATE, "no snapshot taken");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipMemcpyAsync(c->arena, c->snapshot, c->stride * (uint64_t)c->n, hipMemcpyDeviceToDevice, c->stream));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    return SAR_OK;
+}
+
+int sar_ranks_identical(sar_ctx* c, uint64_t elems, int* identical) {
+    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!identical || elems > c->elems()) return set_error(SAR_EINVAL, "bad argument");
+    SAR_HIP(hipSetDevice(c->device));
+    int zero = 0;
+    SAR_HIP(hipMemcpyAsync(c->d_flag, &zero, sizeof(int), hipMemcpyHostToDevice, c->stream));
+    for (int r = 1; r < c->n; ++r)
+        SAR_HIP(sar::launch_compare(c->stream, c->rank_base(0), c->rank_base(r), elems * (uint64_t)elem_size_of(c->dtype), c->d_flag));
+    int flag = 0;
+    SAR_HIP(hipMemcpyAsync(&flag, c->d_flag, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    *identical = flag ? 0 : 1;
+    return SAR_OK;
+}
+
+int sar_get_tuning(sar_ctx* c, sar_tuning_t* out) {
+    if (!c || !out) return set_error(SAR_EINVAL, "null argument");
+    *out = c->tune; return SAR_OK;
+}
+
+int sar_set_tuning(sar_ctx* c, const sar_tuning_t* in) {
+    if (!c || !in) return set_error(SAR_EINVAL, "null argument");
+    if (!valid_tuning(*in)) return set_error(SAR_EINVAL, "tuning value out of range");
+    c->tune = *in; return SAR_OK;
+}
+
+int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph) {
+    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!main_sched) return set_error(SAR_EINVAL, "main schedule is null");
+    for (const sar_schedule* s : {prework, main_sched}) {
+        if (!s) continue;
+        if (s->s.n != c->n) return set_error(SAR_EINVAL, "schedule and context disagree on the rank count");
+        std::string why = sar::validate(s->s);
+        if (!why.empty()) return set_error(SAR_ESCHED, why);
+    }
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    drop_plan(c);
+    std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
+    int rc;
+    try {
+        if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) { drop_plan(c); return rc; }
+        if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) { drop_plan(c); return rc; }
+    } catch (const std::bad_alloc&) { drop_plan(c); return set_error(SAR_ENOMEM, "out of host memory"); }
+    if (!rows.empty()) {
+        SAR_HIP(hipMalloc((void**)&c->d_ops, rows.size() * sizeof(sar::DevOp)));
+        SAR_HIP(hipMemcpy(c->d_ops, rows.data(), rows.size() * sizeof(sar::DevOp), hipMemcpyHostToDevice));
+    }
+    SAR_HIP(hipMalloc((void**)&c->d_ptrs, (ptrs.size() + 1) * sizeof(char*)));
+    if (!ptrs.empty()) SAR_HIP(hipMemcpy(c->d_ptrs, ptrs.data(), ptrs.size() * sizeof(char*), hipMemcpyHostToDevice));
+
+    sar_stats_t st{};
+    sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
+    if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
+    st.rounds = (int)main_sched->s.rounds.size();
+    for (const auto& r : main_sched->s.rounds) st.ops += (int)r.size();
+    for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
+    for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
+
+    if (use_graph) {
+        // the main rounds as one graph: kernel nodes only (no memset nodes)
+        hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+        if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamBeginCapture: ") + hipGetErrorString(e)); }
+        rc = launch_all(c, c->rounds);
+        e = hipStreamEndCapture(c->stream, &c->graph);
+        if (rc != SAR_OK) { drop_plan(c); return rc; }
+        if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e)); }
+        e = hipGraphInstantiate(&c->graph_exec, c->graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e)); }
+        st.uses_graph = 1;
+    }
+    c->stats = st;
+    c->prepared = true;
+    return SAR_OK;
+}
+
+int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
+    if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
+    if (!(delay_ms <= kMaxDelayMs)) return set_error(SAR_EINVAL, "delay out of range");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipEventRecord(c->ev_start, c->stream));
+    if (delay_ms >= 0) {
+        // the straggler's stream is busy for delay_ms while the others do their pre-work
+        const uint64_t ticks = (uint64_t)((double)delay_ms * (double)c->wall_khz);
+        SAR_HIP(hipStreamWaitEvent(c->straggler_stream, c->ev_start, 0));
+        SAR_HIP(sar::launch_sleep(c->straggler_stream, ticks));
+        SAR_HIP(hipEventRecord(c->ev_join, c->straggler_stream));
+        int rc = launch_all(c, c->prework); if (rc) return rc;
+        SAR_HIP(hipStreamWaitEvent(c->stream, c->ev_join, 0));
+    }
+    if (c->graph_exec) SAR_HIP(hipGraphLaunch(c->graph_exec, c->stream));
+    else { int rc = launch_all(c, c->rounds); if (rc) return rc; }
+    SAR_HIP(hipEventRecord(c->ev_stop, c->stream));
+    SAR_HIP(hipEventSynchronize(c->ev_stop));
+    if (delay_ms >= 0) SAR_HIP(hipStreamSynchronize(c->straggler_stream));
+    float ms = 0.f;
+    SAR_HIP(hipEventElapsedTime(&ms, c->ev_start, c->ev_stop));
+    if (elapsed_ms) *elapsed_ms = ms;
+    return SAR_OK;
+}
+
+int sar_run_profiled(sar_ctx* c, float* ms, int cap, int* count) {
+    if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
+    if (cap < 0 || (cap > 0 && !ms)) return set_error(SAR_EINVAL, "bad argument");
+    SAR_HIP(hipSetDevice(c->device));
+    std::vector<const Launch*> ls;
+    for (const auto& L : c->rounds) if (L.total_tiles) ls.push_back(&L);
+    while (c->ev_prof.size() < ls.size() + 1) {
+        hipEvent_t e; SAR_HIP(hipEventCreate(&e)); c->ev_prof.push_back(e);
+    }
+    SAR_HIP(hipEventRecord(c->ev_prof[0], c->stream));
+    for (size_t i = 0; i < ls.size(); ++i) {
+        int rc = launch_one(c, *ls[i]); if (rc) return rc;
+        SAR_HIP(hipEventRecord(c->ev_prof[i + 1], c->stream));
+    }
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    for (size_t i = 0; i < ls.size() && (int)i < cap; ++i) SAR_HIP(hipEventElapsedTime(&ms[i], c->ev_prof[i], c->ev_prof[i + 1]));
+    if (count) *count = (int)ls.size();
+    return SAR_OK;
+}
+
+int sar_launch_bytes(sar_ctx* c, uint64_t* bytes, int cap, int* count) {
+    if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
+    if (cap < 0 || (cap > 0 && !bytes)) return set_error(SAR_EINVAL, "bad argument");
+    int k = 0;
+    for (const auto& L : c->rounds) {
+        if (!L.total_tiles) continue;
+        if (k < cap) bytes[k] = L.algorithmic_bytes;
+        ++k;
+    }
+    if (count) *count = k;
+    return SAR_OK;
+}
+
+int sar_sleep_ticks(sar_ctx* c, float delay_ms, int64_t* ticks) {
+    if (!c || !ticks) return set_error(SAR_EINVAL, "null argument");
+    if (!(delay_ms >= 0) || !(delay_ms <= kMaxDelayMs)) return set_error(SAR_EINVAL, "delay out of range");
+    *ticks = (int64_t)((double)delay_ms * (double)c->wall_khz);
+    return SAR_OK;
+}
+
+int sar_stats(sar_ctx* c, sar_stats_t* out) {
+    if (!c || !out) return set_error(SAR_EINVAL, "null argument");
+    if (!c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
+    *out = c->stats; return SAR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,422 @@
+// gfx950 device code of the schedule executor: one batched kernel per
+// schedule round plus the small fill / compare / sleep kernels.
+//
+// The round kernel replaces, for all rows of a round at once, the reference's
+// "ncclSend/ncclRecv into a temp buffer, then reduce_add<<<ceil(count/256),256>>>"
+// (allreduce_8GPU.cu:29-34 and every call site in :60-874).  It is pure
+// streaming work bound by HBM bandwidth: 16-byte accesses per lane, every
+// wavefront touching 1 KiB of consecutive memory per instruction, U
+// independent vectors in flight per lane and stream, one tile per workgroup so
+// that the hardware dispatcher balances rows of different cost.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kernels.hpp"
+
+namespace sar {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+
+// ---- cache-policy aware 16-byte accesses --------------------------------
+template <bool NT>
+__device__ __forceinline__ f4 ld16(const char* p) {
+    const f4* q = reinterpret_cast<const f4*>(p);
+    if (NT) return __builtin_nontemporal_load(q);
+    return *q;
+}
+template <bool NT>
+__device__ __forceinline__ void st16(char* p, f4 v) {
+    f4* q = reinterpret_cast<f4*>(p);
+    if (NT) __builtin_nontemporal_store(v, q);
+    else *q = v;
+}
+
+// ---- element arithmetic ---------------------------------------------------
+// fp32: IEEE add.  fp16: correctly rounded add (same bits as widening to
+// fp32, adding, and narrowing with round-to-nearest-even).  bf16: widen by a
+// shift, fp32 add, round-to-nearest-even narrow, NaN quieted.
+__device__ __forceinline__ uint32_t bf16_round(float f) {
+    uint32_t x = __float_as_uint(f);
+    uint32_t r = (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;
+    uint32_t q = (x >> 16) | 0x40u;
+    return ((x & 0x7fffffffu) > 0x7f800000u) ? q : r;
+}
+__device__ __forceinline__ uint32_t bf16x2_add(uint32_t a, uint32_t b) {
+    float lo = __uint_as_float(a << 16) + __uint_as_float(b << 16);
+    float hi = __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u);
+    return (bf16_round(lo) & 0xffffu) | (bf16_round(hi) << 16);
+}
+
+template <int DT>
+__device__ __forceinline__ f4 add16(f4 a, f4 b) {
+    if (DT == SAR_F32) {
+        return a + b;
+    } else if (DT == SAR_F16) {
+        h8 x = __builtin_bit_cast(h8, a), y = __builtin_bit_cast(h8, b);
+        return __builtin_bit_cast(f4, x + y);
+    } else {
+        u4 x = __builtin_bit_cast(u4, a), y = __builtin_bit_cast(u4, b), r;
+        r.x = bf16x2_add(x.x, y.x); r.y = bf16x2_add(x.y, y.y);
+        r.z = bf16x2_add(x.z, y.z); r.w = bf16x2_add(x.w, y.w);
+        return __builtin_bit_cast(f4, r);
+    }
+}
+
+template <int DT> struct Elem;
+template <> struct Elem<SAR_F32> { typedef float T; };
+template <> struct Elem<SAR_F16> { typedef _Float16 T; };
+template <> struct Elem<SAR_BF16> { typedef uint16_t T; };
+
+template <int DT>
+__device__ __forceinline__ typename Elem<DT>::T add1(typename Elem<DT>::T a, typename Elem<DT>::T b) {
+    if constexpr (DT == SAR_BF16) {
+        float s = __uint_as_float((uint32_t)a << 16) + __uint_as_float((uint32_t)b << 16);
+        return (uint16_t)bf16_round(s);
+    } else {
+        return a + b;
+    }
+}
+
+// ---- one tile of one row ---------------------------------------------------
+// `len` bytes starting at byte `off` of the row, len <= BLOCK*U*16.
+// Full 16-byte vectors are spread over the lanes with a stride of BLOCK
+// vectors; the < 16 trailing bytes of a row are finished element by element.
+
+template <int DT, int U, int BLOCK, bool LNT, bool SNT>
+__device__ __forceinline__ void tile_copy(char* __restrict__ dst, const char* __restrict__ src, uint64_t off, uint32_t len) {
+    const uint32_t nvec = len >> 4;
+    f4 v[U];
+    if (nvec == BLOCK * U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = ld16<LNT>(src + off + ((uint64_t)(threadIdx.x + u * BLOCK) << 4));
+#pragma unroll
+        for (int u = 0; u < U; ++u) st16<SNT>(dst + off + ((uint64_t)(threadIdx.x + u * BLOCK) << 4), v[u]);
+        return;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        uint32_t i = threadIdx.x + u * BLOCK;
+        if (i < nvec) v[u] = ld16<LNT>(src + off + ((uint64_t)i << 4));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        uint32_t i = threadIdx.x + u * BLOCK;
+        if (i < nvec) st16<SNT>(dst + off + ((uint64_t)i << 4), v[u]);
+    }
+    typedef typename Elem<DT>::T T;
+    const uint32_t tail = (len & 15u) / sizeof(T);
+    if (threadIdx.x < tail) {
+        uint64_t o = off + ((uint64_t)nvec << 4) + threadIdx.x * sizeof(T);
+        *reinterpret_cast<T*>(dst + o) = *reinterpret_cast<const T*>(src + o);
+    }
+}
+
+// dst += src  (TWO = false)   or   s = a + b; a <- s; b <- s  (TWO = true; dst = a, src = b)
+template <int DT, int U, int BLOCK, bool TWO, bool LNT, bool SNT0, bool SNT1>
+__device__ __forceinline__ void tile_reduce(char* __restrict__ dst, char* __restrict__ src, uint64_t off, uint32_t len) {
+    const uint32_t nvec = len >> 4;
+    f4 a[U], b[U];
+    if (nvec == BLOCK * U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            uint64_t o = off + ((uint64_t)(threadIdx.x + u * BLOCK) << 4);
+            a[u] = ld16<LNT>(dst + o);
+            b[u] = ld16<LNT>(src + o);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            uint64_t o = off + ((uint64_t)(threadIdx.x + u * BLOCK) << 4);
+            f4 s = add16<DT>(a[u], b[u]);
+            st16<SNT0>(dst + o, s);
+            if (TWO) st16<SNT1>(src + o, s);
+        }
+        return;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        uint32_t i = threadIdx.x + u * BLOCK;
+        if (i < nvec) { a[u] = ld16<LNT>(dst + off + ((uint64_t)i << 4)); b[u] = ld16<LNT>(src + off + ((uint64_t)i << 4)); }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        uint32_t i = threadIdx.x + u * BLOCK;
+        if (i < nvec) {
+            f4 s = add16<DT>(a[u], b[u]);
+            st16<SNT0>(dst + off + ((uint64_t)i << 4), s);
+            if (TWO) st16<SNT1>(src + off + ((uint64_t)i << 4), s);
+        }
+    }
+    typedef typename Elem<DT>::T T;
+    const uint32_t tail = (len & 15u) / sizeof(T);
+    if (threadIdx.x < tail) {
+        uint64_t o = off + ((uint64_t)nvec << 4) + threadIdx.x * sizeof(T);
+        T s = add1<DT>(*reinterpret_cast<T*>(dst + o), *reinterpret_cast<T*>(src + o));
+        *reinterpret_cast<T*>(dst + o) = s;
+        if (TWO) *reinterpret_cast<T*>(src + o) = s;
+    }
+}
+
+// Ring-ordered multi-source reduce.  srcs[0..nsrc) are in the order the ring
+// adds them: acc = srcs[0]; acc = srcs[k] + acc for k = 1..nsrc-1 (the owner's
+// own data comes last).  The result goes to every dsts[0..ndst).
+template <int DT, int U, int BLOCK, bool LNT, bool SNT>
+__device__ __forceinline__ void tile_mreduce(char* const* __restrict__ srcs, uint32_t nsrc, char* const* __restrict__ dsts, uint32_t ndst,
+                                             uint64_t off, uint32_t len) {
+    const uint32_t nvec = len >> 4;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        uint32_t i = threadIdx.x + u * BLOCK;
+        if (i >= nvec) continue;
+        uint64_t o = off + ((uint64_t)i << 4);
+        f4 acc = ld16<LNT>(srcs[0] + o);
+        for (uint32_t k0 = 1; k0 < nsrc; k0 += 8) {
+            f4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) if (k0 + j < nsrc) v[j] = ld16<LNT>(srcs[k0 + j] + o);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) if (k0 + j < nsrc) acc = add16<DT>(v[j], acc);
+        }
+        for (uint32_t d = 0; d < ndst; ++d) st16<SNT>(dsts[d] + o, acc);
+    }
+    typedef typename Elem<DT>::T T;
+    const uint32_t tail = (len & 15u) / sizeof(T);
+    if (threadIdx.x < tail) {
+        uint64_t o = off + ((uint64_t)nvec << 4) + threadIdx.x * sizeof(T);
+        T acc = *reinterpret_cast<const T*>(srcs[0] + o);
+        for (uint32_t k = 1; k < nsrc; ++k) acc = add1<DT>(*reinterpret_cast<const T*>(srcs[k] + o), acc);
+        for (uint32_t d = 0; d < ndst; ++d) *reinterpret_cast<T*>(dsts[d] + o) = acc;
+    }
+}
+
+// Rows whose pointers are not all 16-byte aligned (unpadded buffer sizes):
+// element by element, still coalesced across the wavefront.
+template <int DT, int BLOCK>
+__device__ __forceinline__ void tile_scalar(uint32_t kind, char* p0, char* p1, uint64_t off, uint32_t len) {
+    typedef typename Elem<DT>::T T;
+    const uint32_t n = len / sizeof(T);
+    for (uint32_t e = threadIdx.x; e < n; e += BLOCK) {
+        uint64_t o = off + (uint64_t)e * sizeof(T);
+        if (kind == SAR_OP_COPY) {
+            *reinterpret_cast<T*>(p0 + o) = *reinterpret_cast<const T*>(p1 + o);
+        } else {
+            T s = add1<DT>(*reinterpret_cast<T*>(p0 + o), *reinterpret_cast<T*>(p1 + o));
+            *reinterpret_cast<T*>(p0 + o) = s;
+            if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
+        }
+    }
+}
+
+// Which row and which tile of it a workgroup owns.
+__device__ __forceinline__ void locate(const DevOp* __restrict__ ops, uint32_t nops, uint32_t total_tiles, uint32_t tiles_per_op,
+                                       uint32_t interleave, uint32_t reverse, uint32_t* row, uint32_t* t) {
+    uint32_t tile = reverse ? total_tiles - 1u - blockIdx.x : blockIdx.x;
+    if (tiles_per_op) {                       // every row of the launch has the same length
+        if (interleave) { *row = tile % nops; *t = tile / nops; }
+        else { *row = tile / tiles_per_op; *t = tile - *row * tiles_per_op; }
+    } else {                                  // rows of different length: find the row by its first tile
+        uint32_t lo = 0, hi = nops;
+        while (hi - lo > 1) { uint32_t mid = (lo + hi) >> 1; if (ops[mid].tile_begin <= tile) lo = mid; else hi = mid; }
+        *row = lo; *t = tile - ops[lo].tile_begin;
+    }
+}
+
+// COPY / REDUCE_INTO / XREDUCE rows of one round; one tile of BLOCK*U vectors per workgroup.
+template <int DT, int U, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void round_kernel(const DevOp* __restrict__ ops, uint32_t nops, uint32_t total_tiles,
+                                                       uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse) {
+    uint32_t j, t;
+    locate(ops, nops, total_tiles, tiles_per_op, interleave, reverse, &j, &t);
+    char* const p0 = ops[j].p0;
+    char* const p1 = ops[j].p1;
+    const uint64_t bytes = ops[j].bytes;
+    const uint32_t kind = ops[j].kind, flags = ops[j].flags;
+    constexpr uint64_t tile_bytes = (uint64_t)BLOCK * U * 16u;
+    const uint64_t off = (uint64_t)t * tile_bytes;
+    if (off >= bytes) return;
+    const uint64_t rem = bytes - off;
+    const uint32_t len = rem < tile_bytes ? (uint32_t)rem : (uint32_t)tile_bytes;
+
+    if (!(flags & DEVOP_VEC)) { tile_scalar<DT, BLOCK>(kind, p0, p1, off, len); return; }
+    const bool lnt = flags & DEVOP_LNT, s0 = flags & DEVOP_SNT0, s1 = flags & DEVOP_SNT1;
+    if (kind == SAR_OP_COPY) {
+        if (lnt) { if (s0) tile_copy<DT, U, BLOCK, true, true>(p0, p1, off, len); else tile_copy<DT, U, BLOCK, true, false>(p0, p1, off, len); }
+        else     { if (s0) tile_copy<DT, U, BLOCK, false, true>(p0, p1, off, len); else tile_copy<DT, U, BLOCK, false, false>(p0, p1, off, len); }
+    } else if (kind == SAR_OP_REDUCE_INTO) {
+        if (lnt) { if (s0) tile_reduce<DT, U, BLOCK, false, true, true, true>(p0, p1, off, len); else tile_reduce<DT, U, BLOCK, false, true, false, false>(p0, p1, off, len); }
+        else     { if (s0) tile_reduce<DT, U, BLOCK, false, false, true, true>(p0, p1, off, len); else tile_reduce<DT, U, BLOCK, false, false, false, false>(p0, p1, off, len); }
+    } else {
+        if (lnt) {
+            if (s0) { if (s1) tile_reduce<DT, U, BLOCK, true, true, true, true>(p0, p1, off, len); else tile_reduce<DT, U, BLOCK, true, true, true, false>(p0, p1, off, len); }
+            else    { if (s1) tile_reduce<DT, U, BLOCK, true, true, false, true>(p0, p1, off, len); else tile_reduce<DT, U, BLOCK, true, true, false, false>(p0, p1, off, len); }
+        } else {
+            if (s0) { if (s1) tile_reduce<DT, U, BLOCK, true, false, true, true>(p0, p1, off, len); else tile_reduce<DT, U, BLOCK, true, false, true, false>(p0, p1, off, len); }
+            else    { if (s1) tile_reduce<DT, U, BLOCK, true, false, false, true>(p0, p1, off, len); else tile_reduce<DT, U, BLOCK, true, false, false, false>(p0, p1, off, len); }
+        }
+    }
+}
+
+// MREDUCE rows (the pre-work collectives): the sources themselves provide the
+// memory-level parallelism, so a tile is BLOCK*MR_U vectors with a small MR_U.
+constexpr int MR_U = 2;
+constexpr int MR_BLOCK = 256;
+
+template <int DT>
+__global__ __launch_bounds__(MR_BLOCK) void mreduce_kernel(const DevOp* __restrict__ ops, uint32_t nops, char* const* __restrict__ ptrs,
+                                                            uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse) {
+    uint32_t j, t;
+    locate(ops, nops, total_tiles, tiles_per_op, interleave, reverse, &j, &t);
+    const uint64_t bytes = ops[j].bytes;
+    const uint32_t flags = ops[j].flags, nsrc = ops[j].nsrc, ndst = ops[j].ndst;
+    char* const* srcs = ptrs + ops[j].ptr_off;
+    char* const* dsts = srcs + nsrc;
+    constexpr uint64_t tile_bytes = (uint64_t)MR_BLOCK * MR_U * 16u;
+    const uint64_t off = (uint64_t)t * tile_bytes;
+    if (off >= bytes) return;
+    const uint64_t rem = bytes - off;
+    const uint32_t len = rem < tile_bytes ? (uint32_t)rem : (uint32_t)tile_bytes;
+    if (!(flags & DEVOP_VEC)) {
+        typedef typename Elem<DT>::T T;
+        const uint32_t n = len / sizeof(T);
+        for (uint32_t e = threadIdx.x; e < n; e += MR_BLOCK) {
+            uint64_t o = off + (uint64_t)e * sizeof(T);
+            T acc = *reinterpret_cast<const T*>(srcs[0] + o);
+            for (uint32_t k = 1; k < nsrc; ++k) acc = add1<DT>(*reinterpret_cast<const T*>(srcs[k] + o), acc);
+            for (uint32_t d = 0; d < ndst; ++d) *reinterpret_cast<T*>(dsts[d] + o) = acc;
+        }
+        return;
+    }
+    const bool lnt = flags & DEVOP_LNT, s0 = flags & DEVOP_SNT0;
+    if (lnt) { if (s0) tile_mreduce<DT, MR_U, MR_BLOCK, true, true>(srcs, nsrc, dsts, ndst, off, len); else tile_mreduce<DT, MR_U, MR_BLOCK, true, false>(srcs, nsrc, dsts, ndst, off, len); }
+    else     { if (s0) tile_mreduce<DT, MR_U, MR_BLOCK, false, true>(srcs, nsrc, dsts, ndst, off, len); else tile_mreduce<DT, MR_U, MR_BLOCK, false, false>(srcs, nsrc, dsts, ndst, off, len); }
+}
+
+#define SAR_LAUNCH_ROUND(DT, U, B) \
+    hipLaunchKernelGGL((round_kernel<DT, U, B>), grid, dim3(B), 0, st, ops, nops, total_tiles, tiles_per_op, interleave, reverse)
+
+template <int DT>
+static hipError_t launch_round_dt(int unroll, int block, dim3 grid, hipStream_t st, const DevOp* ops, uint32_t nops,
+                                  uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse) {
+    switch (unroll * 1024 + block) {
+        case 1 * 1024 + 256: SAR_LAUNCH_ROUND(DT, 1, 256); break;
+        case 2 * 1024 + 256: SAR_LAUNCH_ROUND(DT, 2, 256); break;
+        case 4 * 1024 + 256: SAR_LAUNCH_ROUND(DT, 4, 256); break;
+        case 8 * 1024 + 256: SAR_LAUNCH_ROUND(DT, 8, 256); break;
+        case 1 * 1024 + 512: SAR_LAUNCH_ROUND(DT, 1, 512); break;
+        case 2 * 1024 + 512: SAR_LAUNCH_ROUND(DT, 2, 512); break;
+        case 4 * 1024 + 512: SAR_LAUNCH_ROUND(DT, 4, 512); break;
+        case 8 * 1024 + 512: SAR_LAUNCH_ROUND(DT, 8, 512); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_round(int dtype, int unroll, int block, hipStream_t st, const DevOp* ops, uint32_t nops,
+                        uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse) {
+    if (total_tiles == 0) return hipSuccess;
+    dim3 g(total_tiles);
+    switch (dtype) {
+        case SAR_F32: return launch_round_dt<SAR_F32>(unroll, block, g, st, ops, nops, total_tiles, tiles_per_op, interleave, reverse);
+        case SAR_F16: return launch_round_dt<SAR_F16>(unroll, block, g, st, ops, nops, total_tiles, tiles_per_op, interleave, reverse);
+        case SAR_BF16: return launch_round_dt<SAR_BF16>(unroll, block, g, st, ops, nops, total_tiles, tiles_per_op, interleave, reverse);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+uint64_t mreduce_tile_bytes() { return (uint64_t)MR_BLOCK * MR_U * 16u; }
+
+hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t nops, char* const* ptrs,
+                          uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse) {
+    if (total_tiles == 0) return hipSuccess;
+    dim3 g(total_tiles), b(MR_BLOCK);
+    switch (dtype) {
+        case SAR_F32: hipLaunchKernelGGL((mreduce_kernel<SAR_F32>), g, b, 0, st, ops, nops, ptrs, total_tiles, tiles_per_op, interleave, reverse); break;
+        case SAR_F16: hipLaunchKernelGGL((mreduce_kernel<SAR_F16>), g, b, 0, st, ops, nops, ptrs, total_tiles, tiles_per_op, interleave, reverse); break;
+        case SAR_BF16: hipLaunchKernelGGL((mreduce_kernel<SAR_BF16>), g, b, 0, st, ops, nops, ptrs, total_tiles, tiles_per_op, interleave, reverse); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// ---- fills -------------------------------------------------------------------
+
+__device__ __forceinline__ uint16_t narrow16(float f, int dtype) {
+    if (dtype == SAR_F16) { _Float16 h = (_Float16)f; return __builtin_bit_cast(uint16_t, h); }
+    return (uint16_t)bf16_round(f);
+}
+
+// fill_pattern, allreduce_8GPU.cu:41-45
+__global__ void fill_const_kernel(char* dst, uint64_t elems, float value, int dtype) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+    if (dtype == SAR_F32) { float* d = reinterpret_cast<float*>(dst); for (; i < elems; i += stride) d[i] = value; }
+    else { uint16_t h = narrow16(value, dtype); uint16_t* d = reinterpret_cast<uint16_t*>(dst); for (; i < elems; i += stride) d[i] = h; }
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+// mode 0: a + b*k/2^24;  mode 1: a + b*(sum of 12 such k/2^24 - 6)
+__global__ void fill_random_kernel(char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+    for (; i < elems; i += stride) {
+        double v;
+        if (mode == 0) {
+            uint64_t k = mix64(key + (i + 1) * 0x9E3779B97F4A7C15ull) >> 40;
+            v = a + b * ((double)k * 0x1p-24);
+        } else {
+            uint64_t sum = 0;
+            for (uint64_t j = 0; j < 12; ++j) sum += mix64(key + (i * 12 + j + 1) * 0x9E3779B97F4A7C15ull) >> 40;
+            v = a + b * (((double)sum - 6.0 * 0x1p24) * 0x1p-24);
+        }
+        float f = (float)v;
+        if (dtype == SAR_F32) reinterpret_cast<float*>(dst)[i] = f;
+        else reinterpret_cast<uint16_t*>(dst)[i] = narrow16(f, dtype);
+    }
+}
+
+// *differs is raised when rank buffers a and b differ anywhere in their first `bytes` bytes (bytes a multiple of 2)
+__global__ void compare_kernel(const char* a, const char* b, uint64_t bytes, int* differs) {
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint16_t* x = reinterpret_cast<const uint16_t*>(a);
+    const uint16_t* y = reinterpret_cast<const uint16_t*>(b);
+    bool bad = false;
+    for (uint64_t n = bytes >> 1; i < n; i += stride) bad |= (x[i] != y[i]);
+    if (bad) atomicOr(differs, 1);
+}
+
+// gpu_sleep_kernel, allreduce_8GPU.cu:36-39: one lane spins until `ticks` of
+// the constant-rate wall clock have passed.  The clock is monotonic, so the
+// loop always ends; the host bounds `ticks`.
+__global__ void sleep_kernel(uint64_t ticks) {
+    uint64_t start = wall_clock64();
+    while (wall_clock64() - start < ticks) __builtin_amdgcn_s_sleep(64);
+}
+
+hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype) {
+    if (elems == 0) return hipSuccess;
+    uint64_t blocks = (elems + 255) / 256; if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(fill_const_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, dst, elems, value, dtype);
+    return hipGetLastError();
+}
+hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype) {
+    if (elems == 0) return hipSuccess;
+    uint64_t blocks = (elems + 255) / 256; if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(fill_random_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, dst, elems, key, a, b, mode, dtype);
+    return hipGetLastError();
+}
+hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t bytes, int* differs) {
+    if (bytes < 2) return hipSuccess;
+    uint64_t blocks = (bytes / 2 + 255) / 256; if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(compare_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, a, b, bytes, differs);
+    return hipGetLastError();
+}
+hipError_t launch_sleep(hipStream_t st, uint64_t ticks) {
+    hipLaunchKernelGGL(sleep_kernel, dim3(1), dim3(1), 0, st, ticks);
+    return hipGetLastError();
+}
+
+}  // namespace sar

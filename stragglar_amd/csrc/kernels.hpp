@@ -1,0 +1,46 @@
+// Interface between the host executor and the gfx950 device code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sar.h"
+
+namespace sar {
+
+enum : uint32_t {
+    DEVOP_LNT = 1u,    // loads are streaming (nontemporal)
+    DEVOP_SNT0 = 2u,   // stores to p0 (or to every MREDUCE destination) are streaming
+    DEVOP_SNT1 = 4u,   // stores to p1 are streaming (XREDUCE only)
+    DEVOP_VEC = 8u     // every pointer of the row is 16-byte aligned
+};
+
+// One lowered row of a round, read by the kernel through scalar loads.
+struct DevOp {
+    char* p0;             // COPY/REDUCE_INTO: destination; XREDUCE: first side; MREDUCE: unused
+    char* p1;             // COPY/REDUCE_INTO: source; XREDUCE: second side; MREDUCE: unused
+    uint64_t bytes;       // length of the row
+    uint32_t kind;        // SAR_OP_*
+    uint32_t flags;       // DEVOP_*
+    uint32_t tile_begin;  // first tile of this row within its round
+    uint32_t ntiles;
+    uint32_t nsrc;        // MREDUCE: sources, in add order
+    uint32_t ndst;        // MREDUCE: destinations
+    uint32_t ptr_off;     // MREDUCE: index of srcs[0] in the pointer list; dsts follow the srcs
+    uint32_t reserved0;
+    uint64_t reserved1;
+};
+static_assert(sizeof(DevOp) == 64, "DevOp is read as one 64-byte scalar load");
+
+// COPY / REDUCE_INTO / XREDUCE rows: tiles of block*unroll 16-byte vectors
+hipError_t launch_round(int dtype, int unroll, int block, hipStream_t st, const DevOp* ops, uint32_t nops,
+                        uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
+// MREDUCE rows: tiles of mreduce_tile_bytes()
+uint64_t mreduce_tile_bytes();
+hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t nops, char* const* ptrs,
+                          uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
+hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype);
+hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype);
+hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t bytes, int* differs);
+hipError_t launch_sleep(hipStream_t st, uint64_t ticks);
+
+}  // namespace sar
