@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""bench.py -- achieved HBM GB/s of the emulated n-rank AllReduce on one MI355X.
+
+A step is one pass of the hot path: the 8-rank StragglAR schedule over 8 rank
+buffers of 256 MiB fp32 (padded as pad_buffers.py does: 268 441 600 B) that
+are resident in HBM, uniform[-1,1) seeded per rank, pre-work taken as done
+(DELAY = -1 semantics).  Inputs are restored from a device-side snapshot
+before every step, outside the timed region, as the reference re-fills before
+every iteration; each step is timed with HIP events on the executor's stream,
+as the reference times each iteration.
+
+value     = algorithmic bytes of the schedule (16 S) / mean step time
+roofline  = algorithmic bytes per launch / mean launch duration of the round
+            kernel, measured live with an event pair around every launch
+cpu_baseline = the CPU checker (oracle/, a port) executing the same schedule
+            on the host cores of this box, on a bounded sample
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "achieved HBM GB/s (% of roofline) of emulated n-rank AllReduce, 1 MI355X"
+
+
+def load_table(lib, n):
+    """The StragglAR table for n ranks: the synthesized one shipped with the package if
+    present, else the table the reference hard-codes (n = 4, 8)."""
+    path = os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)
+    if os.path.exists(path):
+        with open(path) as f:
+            return lib.parse(f.read(), n), "synthesizer_pow2 %d" % n
+    return lib.builtin("stragglar", n), "allreduce_%dGPU.cu table" % n
+
+
+def cpu_baseline(lib, ctx, n, elems, table_text_rounds, algorithmic_bytes, budget_s=25.0):
+    """Time the CPU checker on the same workload (inputs downloaded from the device)."""
+    import numpy as np
+    from oracle import load_oracle
+    orc = load_oracle()
+    ctx.restore()
+    inputs = [ctx.download(r) for r in range(n)]
+    out = {}
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except Exception:
+        pass
+    cores = min(cores, 16)
+    for label, threads in (("cpu_baseline", 1), ("cpu_baseline_all_cores", cores)):
+        orc.set_threads(threads)
+        times = []
+        t_begin = time.perf_counter()
+        while True:
+            bufs = [x.copy() for x in inputs]
+            t0 = time.perf_counter()
+            orc.stragglar(bufs, table_text_rounds, "f32")
+            times.append(time.perf_counter() - t0)
+            if len(times) >= 3 or time.perf_counter() - t_begin > budget_s / 2:
+                break
+        best = min(times)
+        out[label] = {
+            "value": round(algorithmic_bytes / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "%d full pass(es) of the same workload (n=%d, %d fp32 elements per rank), best of %d, %.2f s each"
+                      % (len(times), n, elems, len(times), best),
+        }
+    orc.set_threads(1)
+    return out, bufs
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--ranks", type=int, default=8)
+    ap.add_argument("--mib", type=int, default=256, help="unpadded MiB per rank")
+    ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build emulates all ranks on ONE GPU; --gpus %d is not supported (no collectives, "
+              "no second device).  Run with --gpus 1." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import stragglar_amd as sa
+    lib = sa.load_library()           # raises if the HIP library is not built: no fallback
+    n, dtype = args.ranks, "f32"
+    nbytes = lib.pad_bytes(args.mib << 20, n)
+    elems = nbytes // 4
+    ctx = lib.context(0)              # raises without a usable device
+    ctx.alloc_ranks(n, nbytes, dtype)
+    for r in range(n):
+        ctx.fill_uniform(r, 1000 + r, -1.0, 1.0)
+    ctx.snapshot()
+    if args.alg == "stragglar":
+        main_sched, table_name = load_table(lib, n)
+    else:
+        main_sched, table_name = lib.builtin(args.alg, n), args.alg
+    ctx.prepare(main_sched, None, use_graph=not args.no_graph)
+    st = ctx.stats()
+    tune = ctx.get_tuning().as_dict()
+
+    for _ in range(args.warmup):
+        ctx.restore()
+        ctx.run(-1.0)
+    step_ms = []
+    t_wall0 = time.perf_counter()
+    for _ in range(args.steps):
+        ctx.restore()                 # untimed: the batch is put back in place, resident in HBM
+        step_ms.append(ctx.run(-1.0)) # start event, the rounds, stop event, block on stop
+    wall_s = time.perf_counter() - t_wall0
+    identical = ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts)
+    ms = statistics.fmean(step_ms)
+    value = st.algorithmic_bytes / ms / 1e6
+
+    # per-launch durations of the dominant kernel (sar::round_kernel), events on the launch stream
+    launch_bytes = ctx.launch_bytes()
+    per_launch = [0.0] * len(launch_bytes)
+    reps = max(3, min(10, args.steps))
+    ctx.prepare(main_sched, None, use_graph=False)
+    for _ in range(reps):
+        ctx.restore()
+        for i, t in enumerate(ctx.run_profiled()):
+            per_launch[i] += t / reps
+    mean_launch_ms = statistics.fmean(per_launch)
+    mean_launch_bytes = statistics.fmean(launch_bytes)
+    achieved = mean_launch_bytes / mean_launch_ms / 1e6
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "round_kernel_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            t = json.load(f)
+        key = "%s_n%d_%dMiB_f32" % (args.alg, n, args.mib)
+        if key in t:
+            traffic = t[key]["hbm_bytes_per_launch"]
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                "kernel": "sar::round_kernel<f32>", "launches": len(launch_bytes),
+                "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
+    # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
+    rec = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: n=%d %s (%s), %d MiB fp32 per rank padded to %d B, uniform[-1,1) seeded per rank, "
+                               "DELAY=-1, %d ranks resident in one GPU's HBM" % (n, args.alg, table_name, args.mib, nbytes, n),
+                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": not args.no_graph, "tuning": tune},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
+        "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),
+        "ranks_identical_after_run": bool(identical),
+        "roofline": roofline,
+    }
+    if not args.no_cpu and args.alg == "stragglar":
+        from oracle import parse_table
+        gold = os.path.join(ROOT, "tests", "golden", "stragglar_n%d_cu.txt" % n)
+        path = os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)
+        with open(path if os.path.exists(path) else gold) as f:
+            rounds = parse_table(f.read())
+        base, cpu_out = cpu_baseline(lib, ctx, n, elems, rounds, st.algorithmic_bytes)
+        rec.update(base)
+        # the timed GPU result against the checker's, bit for bit, at the full size
+        import numpy as np
+        ctx.restore()
+        ctx.run(-1.0)
+        ok = all(np.array_equal(ctx.download(r).view(np.uint32), cpu_out[r].view(np.uint32)) for r in range(n))
+        rec["bit_exact_vs_cpu_checker"] = bool(ok)
+    ctx.close()
+    print(json.dumps(rec))
+    if not identical or rec.get("bit_exact_vs_cpu_checker") is False:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

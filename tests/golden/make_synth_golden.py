@@ -22,7 +22,9 @@ Two facts of the reference this script has to accommodate:
 
 Usage:  python tests/golden/make_synth_golden.py [/root/reference]
 """
+import contextlib
 import importlib.util
+import io
 import os
 import sys
 
@@ -57,6 +59,12 @@ def main():
         with open(os.path.join(HERE, "synth_pow2_n%d.txt" % n), "w") as f:
             f.write(render(sched))
         print("pow2 n=%d rounds=%d" % (n, len(sched)))
+    # the complete printed table (holdings, active chunks, dashes) for one size of each script
+    buf = io.StringIO()
+    with contextlib.redirect_stdout(buf):
+        pow2.construct_schedule([pow2.GPU(i, 8) for i in range(8)], print_result=True)
+    with open(os.path.join(HERE, "synth_pow2_n8_stdout.txt"), "w") as f:
+        f.write(buf.getvalue())
     try:
         gpus = [pow2.GPU(i, 4) for i in range(4)]
         pow2.construct_schedule(gpus)
@@ -72,6 +80,12 @@ def main():
             f.write("# networkx %s\n" % networkx.__version__)
             f.write(render(sched))
         print("nonpow2 n=%d rounds=%d" % (n, len(sched)))
+    npow2.n = 6
+    buf = io.StringIO()
+    with contextlib.redirect_stdout(buf):
+        npow2.construct_schedule([npow2.GPU(i, 6) for i in range(6)], print_result=True)
+    with open(os.path.join(HERE, "synth_nonpow2_n6_stdout.txt"), "w") as f:
+        f.write(buf.getvalue())
 
 
 if __name__ == "__main__":

@@ -80,3 +80,363 @@ def test_config1_n4_1mib_fp32(gpu_ctx, sarlib, oracle):
         # within 1e-6 relative of an order-independent float64 sum (scaled by the sum of magnitudes)
         scale = np.sum([np.abs(from_bits(x, dtype)) for x in inputs], axis=0)
         assert np.all(np.abs(got[r].astype(np.float64) - total) <= 1e-6 * np.maximum(scale, 1e-30))
+
+
+def shipped_table(n):
+    import os
+    from conftest import ROOT
+    with open(os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)) as f:
+        return f.read()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_config4_shape_n6_nonpow2_with_prework(gpu_ctx, sarlib, oracle, dtype):
+    """BASELINE config 4 at a size the checker finishes quickly: n=6 table from the non-power-of-two
+    synthesizer, fp16 uniform[-0.5,0.5), padded per pad_buffers.py, ReduceScatter pre-work on ranks 0-4."""
+    n = 6
+    nbytes = sarlib.pad_bytes(1 << 20, n)
+    inputs = make_inputs(n, nbytes // ES[dtype], dtype, seed=4, scale=0.5)
+    mine, ref = shipped_table(n), read_golden("synth_nonpow2_n6.txt")
+    got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, mine, delay=0.0)
+    want = run_oracle(oracle, "stragglar", inputs, dtype, ref, delay=0.0)
+    for r in range(n):
+        assert_bits_equal(got[r], want[r], "rank %d" % r)
+
+
+@pytest.mark.parametrize("n,table", [(12, "synth_nonpow2_n12.txt"), (16, "synth_pow2_n16.txt"), (32, "synth_pow2_n32.txt")])
+def test_larger_rank_counts(gpu_ctx, sarlib, oracle, n, table):
+    nbytes = sarlib.pad_bytes(64 << 10, n)
+    inputs = make_inputs(n, nbytes // 4, "f32", seed=n)
+    got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, "f32", read_golden(table), delay=0.0)
+    want = run_oracle(oracle, "stragglar", inputs, "f32", read_golden(table), delay=0.0)
+    for r in range(n):
+        assert_bits_equal(got[r], want[r], "n=%d rank %d" % (n, r))
+    if n == 16:
+        for alg in ("ring", "rhd", "direct"):
+            g = run_gpu(gpu_ctx, sarlib, alg, n, inputs, "f32", None, delay=0.0)
+            w = run_oracle(oracle, alg, inputs, "f32", None, delay=0.0)
+            for r in range(n):
+                assert_bits_equal(g[r], w[r], "%s n=16 rank %d" % (alg, r))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 8 * 7 * 4 * 13 + 5])
+def test_ragged_and_unaligned_sizes(gpu_ctx, sarlib, oracle, elems, dtype):
+    """Sizes that do not divide by n-1 or n (the tail is never moved, chunk = size/(n-1) as in the
+    reference), chunks that are not 16-byte aligned (element-wise path), and buffers shorter than the
+    number of chunks (nothing to move)."""
+    n = 8
+    inputs = make_inputs(n, elems, dtype, seed=elems, kind="normal", scale=3.0)
+    for alg in ("stragglar", "ring", "rhd", "direct"):
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0)
+        want = run_oracle(oracle, alg, inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s elems=%d %s rank %d" % (alg, elems, dtype, r))
+
+
+def test_special_values(gpu_ctx, sarlib, oracle):
+    """Subnormals, signed zeros, infinities and overflow to infinity behave as on the host."""
+    n = 4
+    for dtype in ("f32", "f16", "bf16"):
+        elems = 3 * 256
+        rng = np.random.default_rng(5)
+        inputs = []
+        for r in range(n):
+            x = rng.standard_normal(elems).astype(np.float32)
+            x[0:64] *= np.float32({"f32": 1e-41, "f16": 1e-7, "bf16": 1e-40}[dtype])     # subnormal range
+            x[64:96] = [0.0, -0.0] * 16
+            x[96:128] = np.float32({"f32": 3e38, "f16": 6e4, "bf16": 3e38}[dtype]) * (1 if r % 2 == 0 else 1)
+            x[128:132] = [np.inf, -np.inf, np.inf, 1.0] if r == 0 else [1.0, 1.0, -np.inf if r == 1 else 2.0, np.inf]
+            inputs.append(__import__("oracle").to_bits(x, dtype))
+        got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0)
+        want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n4_cu.txt"), delay=0.0)
+        for r in range(n):
+            if dtype == "f32":
+                assert_bits_equal(got[r], want[r], "%s rank %d" % (dtype, r))
+            else:
+                g, w = from_bits(got[r], dtype), from_bits(want[r], dtype)
+                nan = np.isnan(g) & np.isnan(w)
+                assert np.array_equal(got[r][~nan], want[r][~nan]), (dtype, r)
+
+
+def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
+    n, dtype = 8, "f32"
+    nbytes = sarlib.pad_bytes(300000, n) + 4 * 3          # a partial last tile and a 3-element tail
+    inputs = make_inputs(n, nbytes // 4, dtype, seed=9)
+    want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+    default = gpu_ctx.get_tuning().as_dict()
+    try:
+        for block in (256, 512):
+            for unroll in (1, 2, 4, 8):
+                for order in (0, 1):
+                    for policy, rev in ((0, 0), (1, 1), (2, 1), (2, 0)):
+                        t = dict(block=block, unroll=unroll, order=order, cache_policy=policy, reuse_rounds=2, reverse_odd=rev)
+                        got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
+                        for r in range(n):
+                            assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
+    finally:
+        gpu_ctx.set_tuning(**default)
+
+
+def test_graph_replays_match_eager(gpu_ctx, sarlib, oracle):
+    """The captured graph holds kernel nodes only; every replay, with eager work and synchronisation
+    between replays, must equal the eager result."""
+    n, dtype = 8, "bf16"
+    nbytes = sarlib.pad_bytes(1 << 20, n)
+    inputs = make_inputs(n, nbytes // 2, dtype, seed=10, kind="normal", scale=1e-3)
+    want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, nbytes, dtype)
+    ctx.prepare(sarlib.builtin("stragglar", n), sarlib.builtin("prework_rs", n), use_graph=True)
+    assert ctx.stats().uses_graph == 1
+    for rep in range(4):
+        for r, x in enumerate(inputs):
+            ctx.upload(r, x)                     # eager copies + synchronisation between replays
+        ctx.run(0.0)
+        for r in range(n):
+            assert_bits_equal(ctx.download(r), want[r], "replay %d rank %d" % (rep, r))
+        ctx.fill_const(0, 1.0)                   # unrelated eager kernel before the next replay
+
+
+def test_delay_mode(gpu_ctx, sarlib, oracle):
+    """DELAY >= 0: the straggler's stream sleeps while the pre-work runs; the elapsed time covers the
+    delay (allreduce_8GPU.cu:876-898) and the result is the same as without it."""
+    n, dtype = 8, "f32"
+    nbytes = sarlib.pad_bytes(1 << 20, n)
+    inputs = make_inputs(n, nbytes // 4, dtype, seed=12)
+    want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=5.0)
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, nbytes, dtype)
+    ctx.prepare(sarlib.builtin("stragglar", n), sarlib.builtin("prework_rs", n), use_graph=True)
+    for delay in (5.0, 1.0):
+        for r, x in enumerate(inputs):
+            ctx.upload(r, x)
+        ms = ctx.run(delay)
+        assert delay <= ms < delay + 50.0, ms
+        for r in range(n):
+            assert_bits_equal(ctx.download(r), want[r], "delay %g rank %d" % (delay, r))
+    assert ctx.sleep_ticks(5.0) > 0
+
+
+def test_reference_self_check_pattern(gpu_ctx, sarlib, oracle):
+    """The reference's own check: constant fills end as 36.0 (n=8) / 6.0 (n=4) everywhere."""
+    for n, base, expect in ((8, 1, 36.0), (4, 0, 6.0)):
+        for alg in ("stragglar", "ring", "rhd", "direct"):
+            for dtype in ("f32", "f16", "bf16"):
+                nbytes = sarlib.pad_bytes(4096, n) * (n if alg in ("ring", "rhd") else 1)
+                elems = nbytes // ES[dtype]
+                gpu_ctx.alloc_ranks(n, nbytes, dtype)
+                gpu_ctx.fill_reference_pattern(alg, -1.0, base)
+                host = [np.zeros(elems, np.float32 if dtype == "f32" else np.uint16) for _ in range(n)]
+                oracle.fill_reference_pattern(host, alg, -1.0, base, dtype)
+                for r in range(n):
+                    assert_bits_equal(gpu_ctx.download(r), host[r], "fill %s n=%d rank %d" % (alg, n, r))
+                gpu_ctx.prepare(sarlib.builtin(alg, n), None, use_graph=False)
+                gpu_ctx.run(-1.0)
+                for r in range(n):
+                    assert np.all(from_bits(gpu_ctx.download(r), dtype) == expect), (alg, n, dtype, r)
+                assert gpu_ctx.ranks_identical()
+
+
+def np_uniform(seed, rank, elems, lo, hi):
+    """numpy restatement of sar_fill_uniform: lo + (hi-lo)*k/2^24, k = top 24 bits of a 64-bit mix."""
+    M = (1 << 64) - 1
+    key = (seed * 0xD1B54A32D192ED03 + (rank + 1) * 0x8CB92BA72F3D8DD7) & M
+    i = np.arange(1, elems + 1, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        z = np.uint64(key) + i * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    k = (z >> np.uint64(40)).astype(np.float64)
+    return (lo + (hi - lo) * (k * 2.0 ** -24)).astype(np.float32)
+
+
+def test_seeded_fills(gpu_ctx, sarlib):
+    n = 4
+    elems = 100003
+    gpu_ctx.alloc_ranks(n, elems * 4, "f32")
+    for r in range(n):
+        gpu_ctx.fill_uniform(r, 42, -1.0, 1.0)
+        got = gpu_ctx.download(r)
+        assert_bits_equal(got, np_uniform(42, r, elems, -1.0, 1.0), "uniform rank %d" % r)
+        assert -1.0 <= got.min() and got.max() < 1.0 and abs(float(got.mean())) < 0.02
+    a = gpu_ctx.download(0)
+    gpu_ctx.fill_uniform(0, 43, -1.0, 1.0)
+    assert not np.array_equal(a, gpu_ctx.download(0))
+    gpu_ctx.fill_normal(1, 7, 0.0, 1e-3)
+    g = gpu_ctx.download(1).astype(np.float64)
+    assert abs(g.mean()) < 2e-5 and 0.95e-3 < g.std() < 1.05e-3
+    gpu_ctx.alloc_ranks(n, elems * 2, "bf16")
+    gpu_ctx.fill_uniform(2, 42, -0.5, 0.5)
+    from oracle import to_bits
+    assert_bits_equal(gpu_ctx.download(2), to_bits(np_uniform(42, 2, elems, -0.5, 0.5), "bf16"), "bf16 uniform")
+    gpu_ctx.alloc_ranks(n, elems * 2, "f16")
+    gpu_ctx.fill_uniform(3, 42, -0.5, 0.5)
+    assert_bits_equal(gpu_ctx.download(3), to_bits(np_uniform(42, 3, elems, -0.5, 0.5), "f16"), "f16 uniform")
+
+
+def test_snapshot_restore_and_compare(gpu_ctx, sarlib):
+    n = 4
+    nbytes = sarlib.pad_bytes(1 << 16, n)
+    gpu_ctx.alloc_ranks(n, nbytes, "f32")
+    for r in range(n):
+        gpu_ctx.fill_uniform(r, 1, -1.0, 1.0)
+    before = [gpu_ctx.download(r) for r in range(n)]
+    gpu_ctx.snapshot()
+    assert not gpu_ctx.ranks_identical()
+    gpu_ctx.prepare(sarlib.builtin("ring", n), None, use_graph=False)
+    gpu_ctx.run(-1.0)
+    assert gpu_ctx.ranks_identical()
+    gpu_ctx.fill_const(2, 5.0, elem_off=nbytes // 4 - 1, elems=1)
+    assert not gpu_ctx.ranks_identical()
+    assert gpu_ctx.ranks_identical(nbytes // 4 - 1)
+    gpu_ctx.restore()
+    for r in range(n):
+        assert_bits_equal(gpu_ctx.download(r), before[r])
+
+
+def test_error_paths(gpu_ctx, sarlib):
+    import stragglar_amd as sa
+    ctx = sarlib.context(0)
+    try:
+        with pytest.raises(sa.SarError) as ei:
+            ctx.run(-1.0)
+        assert ei.value.code == -7
+        with pytest.raises(sa.SarError):
+            ctx.prepare(sarlib.builtin("ring", 8))            # no ranks yet
+        ctx.alloc_ranks(4, 4096, "f32")
+        with pytest.raises(sa.SarError) as ei:
+            ctx.prepare(sarlib.builtin("ring", 8))            # rank count mismatch
+        assert ei.value.code == -1
+        bad = sarlib.parse("Round 0\n1 ['StragglerMatching: 0 <-> 3, chunk_id: 0']\n", 4)
+        with pytest.raises(sa.SarError) as ei:
+            ctx.prepare(bad)
+        assert ei.value.code == -6
+        with pytest.raises(sa.SarError):
+            ctx.upload(0, np.zeros(2048, np.float32))          # larger than the rank buffer
+        with pytest.raises(sa.SarError):
+            ctx.upload(4, np.zeros(4, np.float32))
+        with pytest.raises(sa.SarError):
+            ctx.alloc_ranks(4, 4098, "f32")
+        with pytest.raises(sa.SarError):
+            ctx.set_tuning(block=333)
+        ctx.prepare(sarlib.builtin("ring", 4))
+        with pytest.raises(sa.SarError):
+            ctx.run(1e9)
+    finally:
+        ctx.close()
+
+
+def gather_slices(ctx, rank, chunk, parts, offs, length):
+    """The same `length` elements at each offset of every chunk of one rank, downloaded piecewise."""
+    es = ES[ctx.dtype]
+    return np.concatenate([ctx.download(rank, (c * chunk + o) * es, length * es) for c in range(parts) for o in offs])
+
+
+def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle):
+    """BASELINE config 2 at its real size: n=8, 256 MiB fp32 per rank (2 GiB resident), uniform[-1,1)
+    seeded per rank, stragglar (both tables) / ring / rhd / direct on the same inputs.  Every op is
+    element-wise within chunk structure, so parity is checked on a mini problem gathered from the
+    same positions of every chunk, plus `all ranks identical` over the whole buffers."""
+    n, dtype = 8, "f32"
+    nbytes = sarlib.pad_bytes(256 << 20, n)
+    assert nbytes == 268441600
+    elems = nbytes // 4
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, nbytes, dtype)
+    for r in range(n):
+        ctx.fill_uniform(r, 2000 + r, -1.0, 1.0)
+    ctx.snapshot()
+    L = 4096
+    for alg, table, parts in (("stragglar", read_golden("stragglar_n8_cu.txt"), 7), ("stragglar", shipped_table(8), 7),
+                              ("ring", None, 8), ("rhd", None, 8), ("direct", None, 1)):
+        chunk = elems // parts
+        offs = [0, 12345 * 4, chunk // 2, chunk - L]
+        ctx.restore()
+        mini_in = [gather_slices(ctx, r, chunk, parts, offs, L) for r in range(n)]
+        main = sarlib.parse(table, n) if table else sarlib.builtin(alg, n)
+        # direct runs with its pre-work taken as done: the (n-1)-rank AllReduce cuts the buffer at
+        # size/(n-1) boundaries, which a gathered mini problem does not preserve
+        delay = -1.0 if alg == "direct" else 0.0
+        pre = sarlib.builtin("prework_rs", n) if alg == "stragglar" else None
+        ctx.prepare(main, pre, use_graph=True)
+        ctx.run(delay)
+        assert ctx.ranks_identical((elems // parts) * parts), alg
+        want = run_oracle(oracle, alg, mini_in, dtype, table, delay=delay)
+        for r in (0, 3, 7):
+            got = gather_slices(ctx, r, chunk, parts, offs, L)
+            assert_bits_equal(got, want[r], "%s rank %d" % (alg, r))
+        terms = [mini_in[0], mini_in[n - 1]] if alg == "direct" else mini_in    # direct: ranks 0..n-2 hold the pre-sum already
+        total = np.sum([x.astype(np.float64) for x in terms], axis=0)
+        mag = np.sum([np.abs(x.astype(np.float64)) for x in terms], axis=0)
+        assert np.all(np.abs(got.astype(np.float64) - total) <= 1e-6 * mag)
+
+
+def test_config3_bf16_1gib_with_delay(gpu_ctx, sarlib, oracle):
+    """BASELINE config 3: n=8 x 1 GiB bf16 (padded 1 073 744 896 B), normal(0, 1e-3) seeded per rank,
+    sums accumulated in bf16, straggler rank 7 late by DELAY = 5 ms while ranks 0-6 reduce-scatter."""
+    n, dtype = 8, "bf16"
+    nbytes = sarlib.pad_bytes(1 << 30, n)
+    assert nbytes == 1073744896
+    elems = nbytes // 2
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, nbytes, dtype)
+    for r in range(n):
+        ctx.fill_normal(r, 3000 + r, 0.0, 1e-3)
+    chunk, parts, L = elems // 7, 7, 8192
+    offs = [0, 77777 * 8, chunk // 3, chunk - L]
+    mini_in = [gather_slices(ctx, r, chunk, parts, offs, L) for r in range(n)]
+    ctx.prepare(sarlib.parse(shipped_table(8), n), sarlib.builtin("prework_rs", n), use_graph=True)
+    ms = ctx.run(5.0)
+    assert ms > 5.0
+    assert ctx.ranks_identical()
+    want = run_oracle(oracle, "stragglar", mini_in, dtype, read_golden("synth_pow2_n8.txt"), delay=5.0)
+    for r in (0, 6, 7):
+        assert_bits_equal(gather_slices(ctx, r, chunk, parts, offs, L), want[r], "rank %d" % r)
+    vals = np.stack([from_bits(x, dtype) for x in mini_in])
+    got = from_bits(gather_slices(ctx, 0, chunk, parts, offs, L), dtype)
+    assert np.all(np.abs(got - vals.sum(axis=0)) <= 2.0 ** -7 * 7 * np.abs(vals).sum(axis=0) + 1e-30)
+    ctx.alloc_ranks(2, 4096, "f32")      # give the 8 GiB back before the next test
+
+
+def test_config4_full_size_n6_fp16(gpu_ctx, sarlib, oracle):
+    """BASELINE config 4: n=6 x 64 MiB fp16 (padded 67 112 960 B), uniform[-0.5,0.5), pre-work on ranks 0-4,
+    against the checker on the whole buffers."""
+    n, dtype = 6, "f16"
+    nbytes = sarlib.pad_bytes(64 << 20, n)
+    assert nbytes == 67112960
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, nbytes, dtype)
+    for r in range(n):
+        ctx.fill_uniform(r, 4000 + r, -0.5, 0.5)
+    inputs = [ctx.download(r) for r in range(n)]
+    ctx.prepare(sarlib.parse(shipped_table(6), n), sarlib.builtin("prework_rs", n), use_graph=True)
+    ctx.run(0.0)
+    oracle.set_threads(8)
+    try:
+        want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("synth_nonpow2_n6.txt"), delay=0.0)
+    finally:
+        oracle.set_threads(1)
+    for r in range(n):
+        assert_bits_equal(ctx.download(r), want[r], "rank %d" % r)
+
+
+@pytest.mark.parametrize("nbytes", [4 << 10, 64 << 10, 1 << 20, 16 << 20])
+def test_config5_message_size_sweep(gpu_ctx, sarlib, oracle, nbytes):
+    """BASELINE config 5 (the sizes the checker handles on whole buffers; 256 MiB and 1 GiB are covered
+    by the config 2 and 3 tests): n=8 fp32, four algorithms, graph on and off."""
+    n, dtype = 8, "f32"
+    padded = sarlib.pad_bytes(nbytes, n)
+    inputs = make_inputs(n, padded // 4, dtype, seed=nbytes % 1000)
+    oracle.set_threads(8)
+    try:
+        for alg in ("stragglar", "ring", "rhd", "direct"):
+            want = run_oracle(oracle, alg, inputs, dtype, read_golden("synth_pow2_n8.txt"), delay=-1.0)
+            for graph in (False, True):
+                got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype,
+                              shipped_table(8) if alg == "stragglar" else None, delay=-1.0, use_graph=graph)
+                for r in range(n):
+                    assert_bits_equal(got[r], want[r], "%s %d B graph=%s rank %d" % (alg, padded, graph, r))
+    finally:
+        oracle.set_threads(1)
