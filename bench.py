@@ -84,7 +84,7 @@ def main():
     ap.add_argument("--mib", type=int, default=256, help="unpadded MiB per rank")
     ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build emulates all ranks on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -105,7 +105,7 @@ def main():
         main_sched, table_name = load_table(lib, n)
     else:
         main_sched, table_name = lib.builtin(args.alg, n), args.alg
-    ctx.prepare(main_sched, None, use_graph=not args.no_graph)
+    ctx.prepare(main_sched, None, use_graph=args.graph)
     st = ctx.stats()
     tune = ctx.get_tuning().as_dict()
 
@@ -153,7 +153,7 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: n=%d %s (%s), %d MiB fp32 per rank padded to %d B, uniform[-1,1) seeded per rank, "
                                "DELAY=-1, %d ranks resident in one GPU's HBM" % (n, args.alg, table_name, args.mib, nbytes, n),
-                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": not args.no_graph, "tuning": tune},
+                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph), "tuning": tune},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
         "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),

@@ -86,6 +86,9 @@ typedef struct sar_tuning_t {
                           /*     streaming unless the data is read again within `reuse_rounds`       */
     int32_t reuse_rounds; /* look-ahead of policy 2, in rounds                                       */
     int32_t reverse_odd;  /* 1 = odd rounds walk their tiles backwards (keeps the cache tail warm)   */
+    int32_t segments;     /* >1: cut every row into this many pieces and run the whole schedule      */
+                          /*     piece by piece (smaller cache footprint between rounds); 0 = choose */
+                          /*     from the size of the widest round                                    */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

@@ -43,7 +43,7 @@ class Stats(ctypes.Structure):
 
 
 class Tuning(ctypes.Structure):
-    _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd")]
+    _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd", "segments")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

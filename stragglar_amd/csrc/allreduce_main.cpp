@@ -16,7 +16,8 @@
 //   --init MODE        reference (default: rank i <- i+base, self-check on) | uniform | normal
 //   --seed S           seed of --init uniform/normal (default 0)
 //   --base B           constant of rank 0 for --init reference (default 1 for n=8, 0 for n=4, as the reference)
-//   --graph 0|1        replay the rounds as one hipGraph (default 1)
+//   --graph 0|1        replay the rounds as one hipGraph instead of launching them one by one (default 0:
+//                      on this software stack a replayed node costs more than an eager launch)
 //   --report           also print algorithmic GB/s and the HBM-roofline fraction to stderr
 #include <cerrno>
 #include <cmath>
@@ -88,7 +89,7 @@ int main(int argc, char* argv[]) {
     int numIters = atoi(argv[3]);
     float sleepTime = (float)atof(argv[4]);
 
-    int numRanks = 8, dtype = SAR_F32, use_graph = 1, base = -1, report = 0;
+    int numRanks = 8, dtype = SAR_F32, use_graph = 0, base = -1, report = 0;
     unsigned long long seed = 0;
     std::string schedule_path, init = "reference";
     for (int i = 5; i < argc; ++i) {

@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 2, 0, 2, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0};
 
     // prepared plan
     bool prepared = false;
@@ -156,6 +156,23 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
         return false;
     };
 
+    // With segments > 1 every row is cut into that many consecutive pieces and the whole schedule is run
+    // piece by piece: all rounds on the first piece of every chunk, then all rounds on the second, ...
+    // (the work is element-wise, so the pieces are independent); this shrinks what has to stay in the
+    // Infinity Cache between a round and the next.
+    uint64_t nseg = (uint64_t)std::max(0, c->tune.segments);
+    if (nseg == 0) {
+        // automatic: keep the bytes the rows of one round cover near the capacity of the 256 MB cache
+        // (measured on n=8: 1 piece is best at 38 MB rows, 4 pieces at 153 MB rows)
+        uint64_t widest = 0;
+        for (const auto& round : s.rounds) {
+            uint64_t sum = 0;
+            for (const auto& op : round) sum += sar::lower_range(s, op, elems).len * es;
+            widest = std::max(widest, sum);
+        }
+        nseg = std::max<uint64_t>(1, std::min<uint64_t>(256, widest / 300000000ull));
+    }
+    for (uint64_t seg = 0; seg < nseg; ++seg)
     for (size_t ri = 0; ri < own_rounds; ++ri) {
       const auto& round = s.rounds[ri];
       for (int cls = 0; cls < 2; ++cls) {
@@ -166,10 +183,30 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
             const sar::Op& op = round[oi];
             if ((op.kind == SAR_OP_MREDUCE) != (cls != 0)) continue;
             sar::Range rg = sar::lower_range(s, op, elems);
-            uint64_t bytes = rg.len * es;
-            if (bytes == 0) continue;   // buffer shorter than `parts` elements: nothing to move
-            uint64_t doff = rg.dst_off * es, soff = rg.src_off * es;
-            if (doff + bytes > c->bytes_per_rank || soff + bytes > c->bytes_per_rank) return set_error(SAR_ESCHED, "row leaves the rank buffer");
+            const uint64_t row_bytes = rg.len * es;
+            if (row_bytes == 0) continue;   // buffer shorter than `parts` elements: nothing to move
+            const uint64_t row_doff = rg.dst_off * es, row_soff = rg.src_off * es;
+            if (row_doff + row_bytes > c->bytes_per_rank || row_soff + row_bytes > c->bytes_per_rank) return set_error(SAR_ESCHED, "row leaves the rank buffer");
+            // The part of this row that belongs to piece `seg`.  Pieces partition the offset WITHIN a chunk
+            // (rows move whole chunks, so an element only ever meets elements at its own within-chunk
+            // offset): a row of several chunks contributes one span per chunk.
+            struct Span { uint64_t doff, soff, bytes; };
+            std::vector<Span> spans;
+            if (nseg == 1) {
+                spans.push_back({row_doff, row_soff, row_bytes});
+            } else {
+                const uint64_t chunk_bytes = (elems / (uint64_t)s.parts) * es;
+                const uint64_t piece = ((chunk_bytes + nseg - 1) / nseg + 4095u) & ~(uint64_t)4095u;
+                for (int j = 0; j < op.nchunks; ++j) {
+                    const uint64_t base = (uint64_t)j * chunk_bytes;
+                    const uint64_t len = (j == op.nchunks - 1) ? row_bytes - base : chunk_bytes;   // a to_end row ends with a longer chunk
+                    const uint64_t lo = std::min(seg * piece, len);
+                    const uint64_t hi = (seg == nseg - 1) ? len : std::min((seg + 1) * piece, len);
+                    if (lo < hi) spans.push_back({row_doff + base + lo, row_soff + base + lo, hi - lo});
+                }
+            }
+            for (const Span& sp : spans) {
+            const uint64_t doff = sp.doff, soff = sp.soff, bytes = sp.bytes;
             sar::DevOp d{};
             d.kind = (uint32_t)op.kind; d.bytes = bytes;
             bool aligned = true;
@@ -217,6 +254,7 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
             }
             L.algorithmic_bytes += k * bytes;
             rows.push_back(d); L.nops++;
+            }
         }
         if (L.nops == 0) continue;
         L.total_tiles = (uint32_t)tiles;
@@ -247,7 +285,7 @@ int launch_all(sar_ctx* c, const std::vector<Launch>& v) {
 bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
-           (t.reverse_odd == 0 || t.reverse_odd == 1);
+           (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256;
 }
 
 }  // namespace

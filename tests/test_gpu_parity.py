@@ -169,8 +169,9 @@ def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
         for block in (256, 512):
             for unroll in (1, 2, 4, 8):
                 for order in (0, 1):
-                    for policy, rev in ((0, 0), (1, 1), (2, 1), (2, 0)):
-                        t = dict(block=block, unroll=unroll, order=order, cache_policy=policy, reuse_rounds=2, reverse_odd=rev)
+                    for policy, rev, seg in ((0, 0, 1), (1, 1, 2), (2, 1, 0), (2, 0, 5)):
+                        t = dict(block=block, unroll=unroll, order=order, cache_policy=policy, reuse_rounds=2, reverse_odd=rev,
+                                 segments=seg)
                         got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
                         for r in range(n):
                             assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
@@ -440,3 +441,25 @@ def test_config5_message_size_sweep(gpu_ctx, sarlib, oracle, nbytes):
                     assert_bits_equal(got[r], want[r], "%s %d B graph=%s rank %d" % (alg, padded, graph, r))
     finally:
         oracle.set_threads(1)
+
+
+@pytest.mark.parametrize("alg", ["stragglar", "ring", "rhd", "direct"])
+def test_segmented_execution(gpu_ctx, sarlib, oracle, alg):
+    """Running the schedule piece by piece (pieces partition the offset within a chunk, also for rows of
+    several chunks and for the longer last chunk of a whole-buffer row) gives the same bits."""
+    n, dtype = 8, "f32"
+    nbytes = sarlib.pad_bytes(3 << 20, n) * 8 + 24          # divisible by 7 and 8 chunks, plus a ragged tail
+    inputs = make_inputs(n, nbytes // 4, dtype, seed=31)
+    oracle.set_threads(8)
+    try:
+        want = run_oracle(oracle, alg, inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+    finally:
+        oracle.set_threads(1)
+    default = gpu_ctx.get_tuning().as_dict()
+    try:
+        for seg in (2, 3, 7, 16):
+            got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0, tuning=dict(segments=seg))
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "%s segments=%d rank %d" % (alg, seg, r))
+    finally:
+        gpu_ctx.set_tuning(**default)
