@@ -10,8 +10,10 @@ every iteration; each step is timed with HIP events on the executor's stream,
 as the reference times each iteration.
 
 value     = algorithmic bytes of the schedule (16 S) / mean step time
-roofline  = algorithmic bytes per launch / mean launch duration of the round
-            kernel, measured live with an event pair around every launch
+roofline  = algorithmic bytes per launch / mean launch duration of the dominant
+            kernel (the column kernel: one launch per schedule; with
+            --executor 0 the round kernel: one launch per round), measured live
+            with an event pair around every launch
 cpu_baseline = the CPU checker (oracle/, a port) executing the same schedule
             on the host cores of this box, on a bounded sample
 """
@@ -85,6 +87,8 @@ def main():
     ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
+    ap.add_argument("--executor", type=int, default=None, choices=[0, 1],
+                    help="0 = one launch per round, 1 = column executor (one launch per schedule; the library default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build emulates all ranks on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -105,6 +109,8 @@ def main():
         main_sched, table_name = load_table(lib, n)
     else:
         main_sched, table_name = lib.builtin(args.alg, n), args.alg
+    if args.executor is not None:
+        ctx.set_tuning(executor=args.executor)
     ctx.prepare(main_sched, None, use_graph=args.graph)
     st = ctx.stats()
     tune = ctx.get_tuning().as_dict()
@@ -135,16 +141,17 @@ def main():
     mean_launch_bytes = statistics.fmean(launch_bytes)
     achieved = mean_launch_bytes / mean_launch_ms / 1e6
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "round_kernel_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "kernel_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
             t = json.load(f)
-        key = "%s_n%d_%dMiB_f32" % (args.alg, n, args.mib)
+        key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, "column" if tune["executor"] == 1 else "rounds")
         if key in t:
             traffic = t[key]["hbm_bytes_per_launch"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                "kernel": "sar::round_kernel<f32>", "launches": len(launch_bytes),
+                "kernel": "sar::column_kernel<f32, %d>" % tune["col_block"] if tune["executor"] == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
+                "launches": len(launch_bytes),
                 "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
     # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
     rec = {

@@ -89,6 +89,12 @@ typedef struct sar_tuning_t {
     int32_t segments;     /* >1: cut every row into this many pieces and run the whole schedule      */
                           /*     piece by piece (smaller cache footprint between rounds); 0 = choose */
                           /*     from the size of the widest round                                    */
+    int32_t executor;     /* 0 = one launch per round; 1 = column executor: one launch for the whole */
+                          /*     main schedule, each workgroup walking all rounds for its own range  */
+                          /*     of within-chunk offsets (schedules with MREDUCE rows fall back to 0) */
+    int32_t col_wgs;      /* executor 1: resident workgroups per compute unit                        */
+    int32_t col_block;    /* executor 1: threads per workgroup = 16-byte vectors per column (256,    */
+                          /*     512 or 1024)                                                         */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

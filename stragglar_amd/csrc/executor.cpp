@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 1, 4, 512};
 
     // prepared plan
     bool prepared = false;
@@ -65,6 +65,12 @@ struct sar_ctx {
     sar_stats_t stats{};
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
+
+    // column plan (tune.executor == 1): the whole main schedule as one launch
+    bool column = false;
+    uint32_t* d_round_begin = nullptr;
+    uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512;
+    int cu_count = 0;
 
     char* rank_base(int r) const { return arena + (uint64_t)r * stride; }
     uint64_t elems() const { return bytes_per_rank / (uint64_t)elem_size_of(dtype); }
@@ -77,6 +83,8 @@ void drop_plan(sar_ctx* c) {
     if (c->graph) { (void)hipGraphDestroy(c->graph); c->graph = nullptr; }
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
+    if (c->d_round_begin) { (void)hipFree(c->d_round_begin); c->d_round_begin = nullptr; }
+    c->column = false; c->col_rounds = c->col_count = c->col_grid = 0;
     c->prework.clear(); c->rounds.clear(); c->prepared = false;
     c->stats = sar_stats_t{};
 }
@@ -266,6 +274,71 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
     return SAR_OK;
 }
 
+// Column plan: every row of the main schedule, cut into single-chunk rows (all rows then share one
+// within-chunk offset space), in round order, plus the index of each round's first row.
+int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std::vector<uint32_t>& round_begin, uint64_t* widest_row) {
+    const int es = elem_size_of(c->dtype);
+    const uint64_t elems = c->elems();
+    const uint64_t chunk_bytes = (elems / (uint64_t)s.parts) * es;
+    std::vector<std::vector<RowAccess>> acc;
+    for (const auto& round : s.rounds) {
+        std::vector<RowAccess> v;
+        for (const auto& op : round) v.push_back(accesses(s, op, elems, es));
+        acc.push_back(v);
+    }
+    // a column keeps its data close for the whole schedule: anything read again in ANY later round stays cached
+    auto read_later = [&](size_t round, const Touch& t) {
+        for (size_t r = round + 1; r < acc.size(); ++r)
+            for (const auto& ra : acc[r])
+                for (const auto& rd : ra.reads)
+                    if (overlaps(rd, t)) return true;
+        return false;
+    };
+    *widest_row = 0;
+    const size_t first = rows.size();          // round_begin counts from the first column row
+    for (size_t ri = 0; ri < s.rounds.size(); ++ri) {
+        round_begin.push_back((uint32_t)(rows.size() - first));
+        for (size_t oi = 0; oi < s.rounds[ri].size(); ++oi) {
+            const sar::Op& op = s.rounds[ri][oi];
+            if (op.kind == SAR_OP_MREDUCE) return set_error(SAR_ESCHED, "internal: multi-source rows have no column form");
+            sar::Range rg = sar::lower_range(s, op, elems);
+            const uint64_t row_bytes = rg.len * es;
+            if (row_bytes == 0) continue;
+            const uint64_t row_doff = rg.dst_off * es, row_soff = rg.src_off * es;
+            if (row_doff + row_bytes > c->bytes_per_rank || row_soff + row_bytes > c->bytes_per_rank) return set_error(SAR_ESCHED, "row leaves the rank buffer");
+            uint32_t flags = 0;
+            const RowAccess& ra = acc[ri][oi];
+            if (c->tune.cache_policy == 1) {
+                flags = sar::DEVOP_LNT | sar::DEVOP_SNT0 | sar::DEVOP_SNT1;
+            } else if (c->tune.cache_policy == 2) {
+                bool again = false;
+                for (const auto& rd : ra.reads) again |= read_later(ri, rd);
+                if (!again) flags |= sar::DEVOP_LNT;
+                if (!read_later(ri, ra.writes[0])) flags |= sar::DEVOP_SNT0;
+                if (ra.writes.size() > 1 && !read_later(ri, ra.writes[1])) flags |= sar::DEVOP_SNT1;
+            }
+            for (int j = 0; j < op.nchunks; ++j) {
+                const uint64_t base = (uint64_t)j * chunk_bytes;
+                sar::DevOp d{};
+                d.kind = (uint32_t)op.kind;
+                d.bytes = (j == op.nchunks - 1) ? row_bytes - base : chunk_bytes;     // a to_end row ends with a longer chunk
+                d.p0 = c->rank_base(op.dst_rank) + row_doff + base;
+                d.p1 = c->rank_base(op.src_rank) + row_soff + base;
+                d.flags = flags | (((((uintptr_t)d.p0 | (uintptr_t)d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u);
+                *widest_row = std::max(*widest_row, d.bytes);
+                rows.push_back(d);
+            }
+        }
+    }
+    round_begin.push_back((uint32_t)(rows.size() - first));
+    return SAR_OK;
+}
+
+int launch_column_once(sar_ctx* c) {
+    SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->stream, c->d_ops + c->col_first_op, c->d_round_begin, c->col_rounds, c->col_count));
+    return SAR_OK;
+}
+
 int launch_one(sar_ctx* c, const Launch& L) {
     if (L.total_tiles == 0) return SAR_OK;
     const uint32_t interleave = (uint32_t)(c->tune.order == 1);
@@ -282,10 +355,14 @@ int launch_all(sar_ctx* c, const std::vector<Launch>& v) {
     return SAR_OK;
 }
 
+int launch_main(sar_ctx* c) { return c->column ? launch_column_once(c) : launch_all(c, c->rounds); }
+
 bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
-           (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256;
+           (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256 &&
+           (t.executor == 0 || t.executor == 1) && t.col_wgs >= 1 && t.col_wgs <= 64 &&
+           (t.col_block == 256 || t.col_block == 512 || t.col_block == 1024);
 }
 
 }  // namespace
@@ -385,6 +462,8 @@ int sar_create(int device, sar_ctx** out) {
         sar_destroy(c);
         return set_error(SAR_EHIP, std::string("context setup: ") + hipGetErrorString(e));
     }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0) c->cu_count = cus;
     int khz = 0;
     if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0) c->wall_khz = khz;
     *out = c;
@@ -550,10 +629,19 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_plan(c);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
+    std::vector<uint32_t> round_begin; uint32_t col_first = 0; uint64_t widest_row = 0; bool want_column = false;
     int rc;
     try {
         if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) { drop_plan(c); return rc; }
         if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) { drop_plan(c); return rc; }
+        bool columnar = c->tune.executor == 1;
+        for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
+        if (columnar) {
+            col_first = (uint32_t)rows.size();
+            if ((rc = lower_column(c, main_sched->s, rows, round_begin, &widest_row)) != SAR_OK) { drop_plan(c); return rc; }
+            columnar = rows.size() > col_first;
+        }
+        want_column = columnar;
     } catch (const std::bad_alloc&) { drop_plan(c); return set_error(SAR_ENOMEM, "out of host memory"); }
     if (!rows.empty()) {
         SAR_HIP(hipMalloc((void**)&c->d_ops, rows.size() * sizeof(sar::DevOp)));
@@ -562,19 +650,33 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     SAR_HIP(hipMalloc((void**)&c->d_ptrs, (ptrs.size() + 1) * sizeof(char*)));
     if (!ptrs.empty()) SAR_HIP(hipMemcpy(c->d_ptrs, ptrs.data(), ptrs.size() * sizeof(char*), hipMemcpyHostToDevice));
 
+    if (want_column) {
+        SAR_HIP(hipMalloc((void**)&c->d_round_begin, round_begin.size() * sizeof(uint32_t)));
+        SAR_HIP(hipMemcpy(c->d_round_begin, round_begin.data(), round_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        c->col_block = c->tune.col_block;
+        const uint64_t cb = sar::column_bytes(c->col_block);
+        const uint64_t ncols = (widest_row + cb - 1) / cb;
+        if (ncols > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 columns"); }
+        c->col_first_op = col_first; c->col_rounds = (uint32_t)round_begin.size() - 1; c->col_count = (uint32_t)ncols;
+        const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
+        c->col_grid = (uint32_t)std::min<uint64_t>(ncols, resident);
+        c->column = true;
+    }
+
     sar_stats_t st{};
     sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
     if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
     st.rounds = (int)main_sched->s.rounds.size();
     for (const auto& r : main_sched->s.rounds) st.ops += (int)r.size();
-    for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
+    if (c->column) st.launches += 1;
+    else for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
     for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
 
     if (use_graph) {
         // the main rounds as one graph: kernel nodes only (no memset nodes)
         hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
         if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamBeginCapture: ") + hipGetErrorString(e)); }
-        rc = launch_all(c, c->rounds);
+        rc = launch_main(c);
         e = hipStreamEndCapture(c->stream, &c->graph);
         if (rc != SAR_OK) { drop_plan(c); return rc; }
         if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e)); }
@@ -602,7 +704,7 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
         SAR_HIP(hipStreamWaitEvent(c->stream, c->ev_join, 0));
     }
     if (c->graph_exec) SAR_HIP(hipGraphLaunch(c->graph_exec, c->stream));
-    else { int rc = launch_all(c, c->rounds); if (rc) return rc; }
+    else { int rc = launch_main(c); if (rc) return rc; }
     SAR_HIP(hipEventRecord(c->ev_stop, c->stream));
     SAR_HIP(hipEventSynchronize(c->ev_stop));
     if (delay_ms >= 0) SAR_HIP(hipStreamSynchronize(c->straggler_stream));
@@ -616,6 +718,16 @@ int sar_run_profiled(sar_ctx* c, float* ms, int cap, int* count) {
     if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
     if (cap < 0 || (cap > 0 && !ms)) return set_error(SAR_EINVAL, "bad argument");
     SAR_HIP(hipSetDevice(c->device));
+    if (c->column) {
+        while (c->ev_prof.size() < 2) { hipEvent_t e; SAR_HIP(hipEventCreate(&e)); c->ev_prof.push_back(e); }
+        SAR_HIP(hipEventRecord(c->ev_prof[0], c->stream));
+        int rc = launch_column_once(c); if (rc) return rc;
+        SAR_HIP(hipEventRecord(c->ev_prof[1], c->stream));
+        SAR_HIP(hipStreamSynchronize(c->stream));
+        if (cap > 0) SAR_HIP(hipEventElapsedTime(&ms[0], c->ev_prof[0], c->ev_prof[1]));
+        if (count) *count = 1;
+        return SAR_OK;
+    }
     std::vector<const Launch*> ls;
     for (const auto& L : c->rounds) if (L.total_tiles) ls.push_back(&L);
     while (c->ev_prof.size() < ls.size() + 1) {
@@ -636,6 +748,11 @@ int sar_launch_bytes(sar_ctx* c, uint64_t* bytes, int cap, int* count) {
     if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
     if (cap < 0 || (cap > 0 && !bytes)) return set_error(SAR_EINVAL, "bad argument");
     int k = 0;
+    if (c->column) {
+        if (cap > 0) bytes[0] = c->stats.algorithmic_bytes;
+        if (count) *count = 1;
+        return SAR_OK;
+    }
     for (const auto& L : c->rounds) {
         if (!L.total_tiles) continue;
         if (k < cap) bytes[k] = L.algorithmic_bytes;

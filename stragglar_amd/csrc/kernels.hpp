@@ -38,6 +38,12 @@ hipError_t launch_round(int dtype, int unroll, int block, hipStream_t st, const 
 uint64_t mreduce_tile_bytes();
 hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t nops, char* const* ptrs,
                           uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
+// column executor: all rounds of COPY / REDUCE_INTO / XREDUCE rows (each exactly one chunk long) in one
+// launch; rows of round r are ops[round_begin[r] .. round_begin[r+1]); a column is column_bytes(block) wide
+uint64_t column_bytes(int block);
+hipError_t launch_column(int dtype, int block, uint32_t grid, hipStream_t st, const DevOp* ops, const uint32_t* round_begin,
+                         uint32_t nrounds, uint32_t ncols);
+
 hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype);
 hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype);
 hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t bytes, int* differs);

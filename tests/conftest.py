@@ -40,6 +40,7 @@ def gpu_ctx(sarlib):
     """One device context shared by the GPU tests.  Fails (does not skip) when
     no device is usable: the GPU tests must never pass on a fallback."""
     ctx = sarlib.context(0)
+    ctx.default_tuning = ctx.get_tuning().as_dict()
     yield ctx
     ctx.close()
 

@@ -13,11 +13,16 @@ pytestmark = pytest.mark.gpu
 ES = {"f32": 4, "f16": 2, "bf16": 2}
 
 
+@pytest.fixture(autouse=True)
+def _default_tuning(gpu_ctx):
+    gpu_ctx.set_tuning(**gpu_ctx.default_tuning)
+    yield
+
+
 def run_gpu(ctx, sarlib, alg, n, inputs, dtype, table_text=None, delay=-1.0, use_graph=False, tuning=None):
     elems = inputs[0].size
     ctx.alloc_ranks(n, elems * ES[dtype], dtype)
-    if tuning:
-        ctx.set_tuning(**tuning)
+    ctx.set_tuning(**dict(ctx.default_tuning, **(tuning or {})))
     for r, x in enumerate(inputs):
         ctx.upload(r, x)
     prework = None
@@ -46,10 +51,11 @@ def run_oracle(oracle, alg, inputs, dtype, table_text=None, delay=-1.0):
 TABLES = {4: "stragglar_n4_cu.txt", 8: "stragglar_n8_cu.txt"}
 
 
+@pytest.mark.parametrize("executor", [0, 1])
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("alg", ["stragglar", "ring", "rhd", "direct"])
 @pytest.mark.parametrize("n", [4, 8])
-def test_parity_small(gpu_ctx, sarlib, oracle, n, alg, dtype):
+def test_parity_small(gpu_ctx, sarlib, oracle, n, alg, dtype, executor):
     # padded size of pad_buffers.py for 64 KiB: chunks are 1 KiB multiples, divisible by n as well
     nbytes = sarlib.pad_bytes(65536, n)
     while nbytes % (n * ES[dtype] * (n - 1)):
@@ -58,7 +64,8 @@ def test_parity_small(gpu_ctx, sarlib, oracle, n, alg, dtype):
     inputs = make_inputs(n, elems, dtype, seed=7)
     text = read_golden(TABLES[n]) if alg == "stragglar" else None
     for delay in (-1.0, 0.0):
-        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay)
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay, tuning=dict(executor=executor))
+        assert gpu_ctx.stats().launches == (1 if executor == 1 else gpu_ctx.stats().rounds) + (1 if delay >= 0 and alg in ("stragglar", "direct") else 0)
         want = run_oracle(oracle, alg, inputs, dtype, text, delay)
         for r in range(n):
             assert_bits_equal(got[r], want[r], "%s n=%d %s delay=%g rank %d" % (alg, n, dtype, delay, r))
@@ -119,16 +126,17 @@ def test_larger_rank_counts(gpu_ctx, sarlib, oracle, n, table):
                 assert_bits_equal(g[r], w[r], "%s n=16 rank %d" % (alg, r))
 
 
+@pytest.mark.parametrize("executor", [0, 1])
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 8 * 7 * 4 * 13 + 5])
-def test_ragged_and_unaligned_sizes(gpu_ctx, sarlib, oracle, elems, dtype):
+@pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 8 * 7 * 4 * 13 + 5, 7 * 8 * 2051])
+def test_ragged_and_unaligned_sizes(gpu_ctx, sarlib, oracle, elems, dtype, executor):
     """Sizes that do not divide by n-1 or n (the tail is never moved, chunk = size/(n-1) as in the
     reference), chunks that are not 16-byte aligned (element-wise path), and buffers shorter than the
     number of chunks (nothing to move)."""
     n = 8
     inputs = make_inputs(n, elems, dtype, seed=elems, kind="normal", scale=3.0)
     for alg in ("stragglar", "ring", "rhd", "direct"):
-        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0)
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0, tuning=dict(executor=executor))
         want = run_oracle(oracle, alg, inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
         for r in range(n):
             assert_bits_equal(got[r], want[r], "%s elems=%d %s rank %d" % (alg, elems, dtype, r))
@@ -164,19 +172,22 @@ def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
     nbytes = sarlib.pad_bytes(300000, n) + 4 * 3          # a partial last tile and a 3-element tail
     inputs = make_inputs(n, nbytes // 4, dtype, seed=9)
     want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
-    default = gpu_ctx.get_tuning().as_dict()
-    try:
-        for block in (256, 512):
-            for unroll in (1, 2, 4, 8):
-                for order in (0, 1):
-                    for policy, rev, seg in ((0, 0, 1), (1, 1, 2), (2, 1, 0), (2, 0, 5)):
-                        t = dict(block=block, unroll=unroll, order=order, cache_policy=policy, reuse_rounds=2, reverse_odd=rev,
-                                 segments=seg)
-                        got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
-                        for r in range(n):
-                            assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
-    finally:
-        gpu_ctx.set_tuning(**default)
+    for block in (256, 512):
+        for unroll in (1, 2, 4, 8):
+            for order in (0, 1):
+                for policy, rev, seg in ((0, 0, 1), (1, 1, 2), (2, 1, 0), (2, 0, 5)):
+                    t = dict(executor=0, block=block, unroll=unroll, order=order, cache_policy=policy, reuse_rounds=2,
+                             reverse_odd=rev, segments=seg)
+                    got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
+                    for r in range(n):
+                        assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
+    for col_block in (256, 512, 1024):
+        for col_wgs in (1, 4, 16):
+            for policy in (0, 1, 2):
+                t = dict(executor=1, col_block=col_block, col_wgs=col_wgs, cache_policy=policy)
+                got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
+                for r in range(n):
+                    assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
 
 
 def test_graph_replays_match_eager(gpu_ctx, sarlib, oracle):
@@ -335,7 +346,8 @@ def gather_slices(ctx, rank, chunk, parts, offs, length):
     return np.concatenate([ctx.download(rank, (c * chunk + o) * es, length * es) for c in range(parts) for o in offs])
 
 
-def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle):
+@pytest.mark.parametrize("executor", [0, 1])
+def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
     """BASELINE config 2 at its real size: n=8, 256 MiB fp32 per rank (2 GiB resident), uniform[-1,1)
     seeded per rank, stragglar (both tables) / ring / rhd / direct on the same inputs.  Every op is
     element-wise within chunk structure, so parity is checked on a mini problem gathered from the
@@ -345,6 +357,7 @@ def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle):
     assert nbytes == 268441600
     elems = nbytes // 4
     ctx = gpu_ctx
+    ctx.set_tuning(executor=executor)
     ctx.alloc_ranks(n, nbytes, dtype)
     for r in range(n):
         ctx.fill_uniform(r, 2000 + r, -1.0, 1.0)
@@ -435,10 +448,11 @@ def test_config5_message_size_sweep(gpu_ctx, sarlib, oracle, nbytes):
         for alg in ("stragglar", "ring", "rhd", "direct"):
             want = run_oracle(oracle, alg, inputs, dtype, read_golden("synth_pow2_n8.txt"), delay=-1.0)
             for graph in (False, True):
-                got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype,
-                              shipped_table(8) if alg == "stragglar" else None, delay=-1.0, use_graph=graph)
-                for r in range(n):
-                    assert_bits_equal(got[r], want[r], "%s %d B graph=%s rank %d" % (alg, padded, graph, r))
+                for executor in (0, 1):
+                    got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, shipped_table(8) if alg == "stragglar" else None,
+                                  delay=-1.0, use_graph=graph, tuning=dict(executor=executor))
+                    for r in range(n):
+                        assert_bits_equal(got[r], want[r], "%s %d B graph=%s executor=%d rank %d" % (alg, padded, graph, executor, r))
     finally:
         oracle.set_threads(1)
 
@@ -455,11 +469,7 @@ def test_segmented_execution(gpu_ctx, sarlib, oracle, alg):
         want = run_oracle(oracle, alg, inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
     finally:
         oracle.set_threads(1)
-    default = gpu_ctx.get_tuning().as_dict()
-    try:
-        for seg in (2, 3, 7, 16):
-            got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0, tuning=dict(segments=seg))
-            for r in range(n):
-                assert_bits_equal(got[r], want[r], "%s segments=%d rank %d" % (alg, seg, r))
-    finally:
-        gpu_ctx.set_tuning(**default)
+    for seg in (2, 3, 7, 16):
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0, tuning=dict(executor=0, segments=seg))
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s segments=%d rank %d" % (alg, seg, r))
