@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 1, 4, 512};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 1, 64, 512};
 
     // prepared plan
     bool prepared = false;
@@ -361,7 +361,7 @@ bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
            (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256 &&
-           (t.executor == 0 || t.executor == 1) && t.col_wgs >= 1 && t.col_wgs <= 64 &&
+           (t.executor == 0 || t.executor == 1) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
            (t.col_block == 256 || t.col_block == 512 || t.col_block == 1024);
 }
 

@@ -342,17 +342,13 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // ---- column executor: the whole schedule in one launch, no waiting between workgroups -----------
 // Rows move whole chunks, so an element only ever meets the elements at its own offset within a
 // chunk: the schedule falls apart into independent "columns" (one range of within-chunk offsets each).
-// A workgroup owns a column of BLOCK 16-byte vectors and walks ALL rounds for it, one round after the
-// other, with nothing but a workgroup barrier in between.  Every row still performs its own loads and
-// stores on the rank buffers, in schedule order for each element; but what a later round re-reads was
-// written by the same compute unit moments ago and comes from L2 / Infinity Cache instead of HBM.
-// Within a round the rows are independent, so their loads are issued together (COL_ROWS at a time)
-// before the first add or store.
-constexpr int COL_ROWS = 8;
-
-template <bool NT>
-__device__ __forceinline__ f4 ld16p(const char* p, bool pred) { f4 v = {0.f, 0.f, 0.f, 0.f}; if (pred) v = ld16<NT>(p); return v; }
-
+// A workgroup owns a column of BLOCK 16-byte vectors and walks ALL rounds for it, row after row, with
+// nothing but a workgroup barrier between rounds.  Every row still performs its own loads and stores on
+// the rank buffers, in schedule order for each element; but what a later round re-reads was written by
+// the same compute unit moments ago and comes from L2 / Infinity Cache instead of HBM.
+// One row at a time and one vector per lane turned out best (28 VGPRs, eight waves per SIMD resident:
+// the other workgroups of the compute unit cover a row's latency; batching the loads of several rows or
+// several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
 template <int DT, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ round_begin,
                                                         uint32_t nrounds, uint32_t ncols) {
@@ -363,59 +359,40 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
         const uint64_t voff = off + ((uint64_t)threadIdx.x << 4);       // this lane's vector within every row
         for (uint32_t r = 0; r < nrounds; ++r) {
             const uint32_t rb = round_begin[r], re = round_begin[r + 1];
-            for (uint32_t j0 = rb; j0 < re; j0 += COL_ROWS) {
-                f4 a[COL_ROWS], b[COL_ROWS];
-#pragma unroll
-                for (int q = 0; q < COL_ROWS; ++q) {
-                    const uint32_t j = j0 + q;
-                    if (j < re) {
-                        const uint32_t flags = ops[j].flags;
-                        const bool mine = (flags & DEVOP_VEC) && voff + 16u <= ops[j].bytes;
-                        if (flags & DEVOP_LNT) {
-                            b[q] = ld16p<true>(ops[j].p1 + voff, mine);
-                            if (ops[j].kind != SAR_OP_COPY) a[q] = ld16p<true>(ops[j].p0 + voff, mine);
-                        } else {
-                            b[q] = ld16p<false>(ops[j].p1 + voff, mine);
-                            if (ops[j].kind != SAR_OP_COPY) a[q] = ld16p<false>(ops[j].p0 + voff, mine);
-                        }
+            for (uint32_t j = rb; j < re; ++j) {
+                const uint32_t flags = ops[j].flags, kind = ops[j].kind;
+                const uint64_t bytes = ops[j].bytes;
+                char* const p0 = ops[j].p0;
+                char* const p1 = ops[j].p1;
+                if (flags & DEVOP_VEC) {
+                    if (voff + 16u <= bytes) {
+                        f4 a = {0.f, 0.f, 0.f, 0.f}, b;
+                        if (flags & DEVOP_LNT) { b = ld16<true>(p1 + voff); if (kind != SAR_OP_COPY) a = ld16<true>(p0 + voff); }
+                        else                   { b = ld16<false>(p1 + voff); if (kind != SAR_OP_COPY) a = ld16<false>(p0 + voff); }
+                        const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
+                        if (flags & DEVOP_SNT0) st16<true>(p0 + voff, s); else st16<false>(p0 + voff, s);
+                        if (kind == SAR_OP_XREDUCE) { if (flags & DEVOP_SNT1) st16<true>(p1 + voff, s); else st16<false>(p1 + voff, s); }
                     }
-                }
-#pragma unroll
-                for (int q = 0; q < COL_ROWS; ++q) {
-                    const uint32_t j = j0 + q;
-                    if (j < re) {
-                        const uint32_t flags = ops[j].flags, kind = ops[j].kind;
-                        const uint64_t bytes = ops[j].bytes;
-                        char* const p0 = ops[j].p0;
-                        char* const p1 = ops[j].p1;
-                        if (flags & DEVOP_VEC) {
-                            if (voff + 16u <= bytes) {
-                                const f4 s = kind == SAR_OP_COPY ? b[q] : add16<DT>(a[q], b[q]);
-                                if (flags & DEVOP_SNT0) st16<true>(p0 + voff, s); else st16<false>(p0 + voff, s);
-                                if (kind == SAR_OP_XREDUCE) { if (flags & DEVOP_SNT1) st16<true>(p1 + voff, s); else st16<false>(p1 + voff, s); }
-                            }
-                            // the < 16 bytes behind the last whole vector of the row, in the column that holds them
-                            const uint64_t tail_at = bytes & ~(uint64_t)15u;
-                            const uint32_t tail = (uint32_t)(bytes & 15u) / sizeof(T);
-                            if (tail && tail_at >= off && tail_at < off + col_bytes && threadIdx.x < tail) {
-                                const uint64_t o = tail_at + threadIdx.x * sizeof(T);
-                                T s = *reinterpret_cast<const T*>(p1 + o);
-                                if (kind != SAR_OP_COPY) s = add1<DT>(*reinterpret_cast<const T*>(p0 + o), s);
-                                *reinterpret_cast<T*>(p0 + o) = s;
-                                if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
-                            }
-                        } else if (off < bytes) {                       // row not 16-byte aligned: element by element
-                            const uint64_t rem = bytes - off;
-                            const uint32_t len = rem < col_bytes ? (uint32_t)rem : (uint32_t)col_bytes;
-                            tile_scalar<DT, BLOCK>(kind, p0, p1, off, len);
-                        }
+                    // the < 16 bytes behind the last whole vector of the row, in the column that holds them
+                    const uint64_t tail_at = bytes & ~(uint64_t)15u;
+                    const uint32_t tail = (uint32_t)(bytes & 15u) / sizeof(T);
+                    if (tail && tail_at >= off && tail_at < off + col_bytes && threadIdx.x < tail) {
+                        const uint64_t o = tail_at + threadIdx.x * sizeof(T);
+                        T s = *reinterpret_cast<const T*>(p1 + o);
+                        if (kind != SAR_OP_COPY) s = add1<DT>(*reinterpret_cast<const T*>(p0 + o), s);
+                        *reinterpret_cast<T*>(p0 + o) = s;
+                        if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
                     }
+                } else if (off < bytes) {                               // row not 16-byte aligned: element by element
+                    const uint64_t rem = bytes - off;
+                    const uint32_t len = rem < col_bytes ? (uint32_t)rem : (uint32_t)col_bytes;
+                    tile_scalar<DT, BLOCK>(kind, p0, p1, off, len);
                 }
             }
             // This round's stores are complete before this workgroup's loads of the next round.  (Lanes mostly
             // re-read what they wrote themselves, but elements change lanes between aligned and unaligned
             // rows and at partial vectors; measured, the barrier also pays for itself by keeping the waves
-            // of a workgroup on the same rows: 6.8 against 6.3 TB/s without it.)
+            // of a workgroup on the same rows.)
             __syncthreads();
         }
     }

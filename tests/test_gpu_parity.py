@@ -182,7 +182,7 @@ def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
                     for r in range(n):
                         assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
     for col_block in (256, 512, 1024):
-        for col_wgs in (1, 4, 16):
+        for col_wgs in (1, 4, 64, 4096):
             for policy in (0, 1, 2):
                 t = dict(executor=1, col_block=col_block, col_wgs=col_wgs, cache_policy=policy)
                 got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
