@@ -87,8 +87,8 @@ def main():
     ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
-    ap.add_argument("--executor", type=int, default=None, choices=[0, 1],
-                    help="0 = one launch per round, 1 = column executor (one launch per schedule; the library default)")
+    ap.add_argument("--executor", type=int, default=None, choices=[0, 1, 2],
+                    help="0 = one launch per round, 1 = column executor (one launch per schedule), 2 = chosen by the library's cost model (default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build emulates all ranks on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -145,12 +145,12 @@ def main():
     if os.path.exists(tpath):
         with open(tpath) as f:
             t = json.load(f)
-        key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, "column" if tune["executor"] == 1 else "rounds")
+        key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, "column" if st.executor == 1 else "rounds")
         if key in t:
             traffic = t[key]["hbm_bytes_per_launch"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                "kernel": "sar::column_kernel<f32, %d>" % tune["col_block"] if tune["executor"] == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
+                "kernel": "sar::column_kernel<f32, %d>" % st.col_block if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
                 "launches": len(launch_bytes),
                 "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
     # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
@@ -160,7 +160,7 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: n=%d %s (%s), %d MiB fp32 per rank padded to %d B, uniform[-1,1) seeded per rank, "
                                "DELAY=-1, %d ranks resident in one GPU's HBM" % (n, args.alg, table_name, args.mib, nbytes, n),
-                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph), "tuning": tune},
+                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph), "tuning": tune, "executor_used": "column" if st.executor == 1 else "rounds"},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
         "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),

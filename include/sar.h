@@ -75,6 +75,8 @@ typedef struct sar_stats_t {
     int32_t launches;              /* kernel launches per sar_run (main + pre-work, sleep excluded)               */
     int32_t ops;                   /* rows of the main schedule                                                   */
     int32_t uses_graph;            /* 1 if sar_run replays a hipGraph                                             */
+    int32_t executor;              /* executor the main schedule was lowered for: 0 per round, 1 column           */
+    int32_t col_block;             /* column executor: threads per workgroup in use (0 otherwise)                 */
 } sar_stats_t;
 
 /* run-time tunables of the round kernel; sar_get_tuning() reports the defaults */
@@ -91,10 +93,11 @@ typedef struct sar_tuning_t {
                           /*     from the size of the widest round                                    */
     int32_t executor;     /* 0 = one launch per round; 1 = column executor: one launch for the whole */
                           /*     main schedule, each workgroup walking all rounds for its own range  */
-                          /*     of within-chunk offsets (schedules with MREDUCE rows fall back to 0) */
-    int32_t col_wgs;      /* executor 1: resident workgroups per compute unit                        */
-    int32_t col_block;    /* executor 1: threads per workgroup = 16-byte vectors per column (256,    */
-                          /*     512 or 1024)                                                         */
+                          /*     of within-chunk offsets (schedules with MREDUCE rows fall back to   */
+                          /*     0); 2 = whichever a small cost model expects to be faster (default) */
+    int32_t col_wgs;      /* column executor: workgroups per compute unit in the grid                */
+    int32_t col_block;    /* column executor: threads per workgroup = 16-byte vectors per column     */
+                          /*     (256, 512 or 1024; 0 = chosen from the number of columns)           */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

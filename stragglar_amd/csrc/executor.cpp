@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 1, 64, 512};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0};
 
     // prepared plan
     bool prepared = false;
@@ -334,6 +334,26 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
     return SAR_OK;
 }
 
+// Which executor is expected to be faster (executor = 2).  Constants are measurements on MI355X:
+// the column kernel moves 7.1 algorithmic TB/s when there are columns enough to fill the chip and a
+// column is up to ~128 rows long (n = 8), less for longer columns, whose workgroups drift apart and
+// scatter the access streams (6.4 up to 256 rows, 5.3 beyond); a workgroup needs about 0.6 us per row
+// while everything stays cache resident, 0.95 us beyond that; one launch per round moves 6.5 TB/s and
+// costs about 3 us per launch.
+bool column_pays(const sar_ctx* c, size_t column_rows, uint64_t widest_row, int col_block) {
+    const double bytes = (double)c->stats.algorithmic_bytes;
+    const uint64_t cb = sar::column_bytes(col_block);
+    const double ncols = (double)((widest_row + cb - 1) / cb);
+    const double resident = (double)std::max(1, c->cu_count) * (2048.0 / col_block);
+    const double per_row_us = (double)c->stride * c->n <= 200e6 ? 0.6 : 0.95;
+    const double passes = std::ceil(ncols / resident);
+    const double column_rate = column_rows <= 128 ? 7.1e6 : column_rows <= 256 ? 6.4e6 : 5.3e6;      // bytes per us
+    const double est_column = std::max(bytes / column_rate, (double)column_rows * per_row_us * passes) + 4.0;
+    double est_rounds = 0;
+    for (const auto& L : c->rounds) if (L.total_tiles) est_rounds += 3.0 + (double)L.algorithmic_bytes / 6.5e6;
+    return est_column <= est_rounds;
+}
+
 int launch_column_once(sar_ctx* c) {
     SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->stream, c->d_ops + c->col_first_op, c->d_round_begin, c->col_rounds, c->col_count));
     return SAR_OK;
@@ -361,8 +381,8 @@ bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
            (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256 &&
-           (t.executor == 0 || t.executor == 1) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
-           (t.col_block == 256 || t.col_block == 512 || t.col_block == 1024);
+           (t.executor >= 0 && t.executor <= 2) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
+           (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024);
 }
 
 }  // namespace
@@ -629,17 +649,23 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_plan(c);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    std::vector<uint32_t> round_begin; uint32_t col_first = 0; uint64_t widest_row = 0; bool want_column = false;
+    std::vector<uint32_t> round_begin; uint32_t col_first = 0; uint64_t widest_row = 0; bool want_column = false; int col_block = 512;
     int rc;
     try {
         if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) { drop_plan(c); return rc; }
         if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) { drop_plan(c); return rc; }
-        bool columnar = c->tune.executor == 1;
+        sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &c->stats.algorithmic_bytes, nullptr);
+        bool columnar = c->tune.executor != 0;
         for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
         if (columnar) {
             col_first = (uint32_t)rows.size();
             if ((rc = lower_column(c, main_sched->s, rows, round_begin, &widest_row)) != SAR_OK) { drop_plan(c); return rc; }
             columnar = rows.size() > col_first;
+        }
+        if (columnar) {
+            // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
+            col_block = c->tune.col_block ? c->tune.col_block : (widest_row / sar::column_bytes(512) >= 2048 ? 512 : 256);
+            if (c->tune.executor == 2) columnar = column_pays(c, rows.size() - col_first, widest_row, col_block);
         }
         want_column = columnar;
     } catch (const std::bad_alloc&) { drop_plan(c); return set_error(SAR_ENOMEM, "out of host memory"); }
@@ -653,7 +679,7 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     if (want_column) {
         SAR_HIP(hipMalloc((void**)&c->d_round_begin, round_begin.size() * sizeof(uint32_t)));
         SAR_HIP(hipMemcpy(c->d_round_begin, round_begin.data(), round_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
-        c->col_block = c->tune.col_block;
+        c->col_block = (uint32_t)col_block;
         const uint64_t cb = sar::column_bytes(c->col_block);
         const uint64_t ncols = (widest_row + cb - 1) / cb;
         if (ncols > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 columns"); }
@@ -684,6 +710,8 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
         if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e)); }
         st.uses_graph = 1;
     }
+    st.executor = c->column ? 1 : 0;
+    st.col_block = c->column ? (int32_t)c->col_block : 0;
     c->stats = st;
     c->prepared = true;
     return SAR_OK;

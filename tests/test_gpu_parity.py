@@ -65,7 +65,9 @@ def test_parity_small(gpu_ctx, sarlib, oracle, n, alg, dtype, executor):
     text = read_golden(TABLES[n]) if alg == "stragglar" else None
     for delay in (-1.0, 0.0):
         got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay, tuning=dict(executor=executor))
-        assert gpu_ctx.stats().launches == (1 if executor == 1 else gpu_ctx.stats().rounds) + (1 if delay >= 0 and alg in ("stragglar", "direct") else 0)
+        st = gpu_ctx.stats()
+        assert st.executor == executor
+        assert st.launches == (1 if executor == 1 else st.rounds) + (1 if delay >= 0 and alg in ("stragglar", "direct") else 0)
         want = run_oracle(oracle, alg, inputs, dtype, text, delay)
         for r in range(n):
             assert_bits_equal(got[r], want[r], "%s n=%d %s delay=%g rank %d" % (alg, n, dtype, delay, r))
@@ -126,7 +128,7 @@ def test_larger_rank_counts(gpu_ctx, sarlib, oracle, n, table):
                 assert_bits_equal(g[r], w[r], "%s n=16 rank %d" % (alg, r))
 
 
-@pytest.mark.parametrize("executor", [0, 1])
+@pytest.mark.parametrize("executor", [0, 1, 2])
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 8 * 7 * 4 * 13 + 5, 7 * 8 * 2051])
 def test_ragged_and_unaligned_sizes(gpu_ctx, sarlib, oracle, elems, dtype, executor):
