@@ -165,6 +165,14 @@ void sar_destroy(sar_ctx* ctx);
  * arena; rank r starts at r*stride, stride = bytes rounded up to 2 MiB. */
 int sar_alloc_ranks(sar_ctx* ctx, int n, uint64_t bytes_per_rank, int dtype);
 
+/* Use caller-owned device buffers as the rank buffers instead of the arena: device_ptrs[r] is rank r's
+ * buffer of bytes_per_rank bytes on the context's GPU; the buffers must not overlap and stay valid until
+ * the next sar_alloc_ranks / sar_adopt_ranks / sar_destroy; the context never frees them.  This is what
+ * a caller holding one flat gradient tensor per emulated rank needs (the role of tensors[0].data_ptr() in
+ * allreduce_stragglar, implementation/custom_backend/src/dummy.cpp:256-271).  The caller orders its own
+ * work on those buffers against sar_run (which blocks until the result is complete). */
+int sar_adopt_ranks(sar_ctx* ctx, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype);
+
 int sar_upload(sar_ctx* ctx, int rank, uint64_t byte_off, const void* host, uint64_t bytes);
 int sar_download(sar_ctx* ctx, int rank, uint64_t byte_off, void* host, uint64_t bytes);
 

@@ -66,7 +66,7 @@ EXPORTS = [
     "sar_schedule_parse", "sar_schedule_builtin", "sar_schedule_validate", "sar_schedule_ranks",
     "sar_schedule_parts", "sar_schedule_rounds", "sar_schedule_round_ops", "sar_schedule_op",
     "sar_schedule_bytes", "sar_schedule_free",
-    "sar_create", "sar_destroy", "sar_alloc_ranks", "sar_upload", "sar_download", "sar_fill_const",
+    "sar_create", "sar_destroy", "sar_alloc_ranks", "sar_adopt_ranks", "sar_upload", "sar_download", "sar_fill_const",
     "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats",
@@ -103,6 +103,7 @@ class Library:
             "sar_create": (c_int, [c_int, P(vp)]),
             "sar_destroy": (None, [vp]),
             "sar_alloc_ranks": (c_int, [vp, c_int, u64, c_int]),
+            "sar_adopt_ranks": (c_int, [vp, c_int, P(vp), u64, c_int]),
             "sar_upload": (c_int, [vp, c_int, u64, vp, u64]),
             "sar_download": (c_int, [vp, c_int, u64, vp, u64]),
             "sar_fill_const": (c_int, [vp, c_int, u64, u64, ctypes.c_double]),
@@ -243,6 +244,12 @@ class Context:
     def alloc_ranks(self, n: int, bytes_per_rank: int, dtype: str = "f32"):
         self._c(self._lib.lib.sar_alloc_ranks(self._h, n, bytes_per_rank, DTYPES[dtype]))
         self.n, self.dtype, self.bytes_per_rank = n, dtype, bytes_per_rank
+
+    def adopt_ranks(self, device_ptrs: Sequence[int], bytes_per_rank: int, dtype: str = "f32"):
+        """Use caller-owned device buffers (raw addresses, one per rank) as the rank buffers."""
+        arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
+        self._c(self._lib.lib.sar_adopt_ranks(self._h, len(device_ptrs), arr, bytes_per_rank, DTYPES[dtype]))
+        self.n, self.dtype, self.bytes_per_rank = len(device_ptrs), dtype, bytes_per_rank
 
     @property
     def elems(self) -> int:

@@ -72,8 +72,12 @@ struct sar_ctx {
     uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512;
     int cu_count = 0;
 
-    char* rank_base(int r) const { return arena + (uint64_t)r * stride; }
+    std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
+
+    bool has_ranks() const { return arena != nullptr || !adopted.empty(); }
+    char* rank_base(int r) const { return adopted.empty() ? arena + (uint64_t)r * stride : adopted[(size_t)r]; }
     uint64_t elems() const { return bytes_per_rank / (uint64_t)elem_size_of(dtype); }
+    uint64_t snapshot_stride() const { return adopted.empty() ? stride : (bytes_per_rank + 255u) & ~(uint64_t)255u; }
 };
 
 namespace {
@@ -93,6 +97,7 @@ void drop_ranks(sar_ctx* c) {
     drop_plan(c);
     if (c->arena) { (void)hipFree(c->arena); c->arena = nullptr; }
     if (c->snapshot) { (void)hipFree(c->snapshot); c->snapshot = nullptr; }
+    c->adopted.clear();
     c->n = 0; c->bytes_per_rank = 0; c->stride = 0;
 }
 
@@ -345,7 +350,7 @@ bool column_pays(const sar_ctx* c, size_t column_rows, uint64_t widest_row, int 
     const uint64_t cb = sar::column_bytes(col_block);
     const double ncols = (double)((widest_row + cb - 1) / cb);
     const double resident = (double)std::max(1, c->cu_count) * (2048.0 / col_block);
-    const double per_row_us = (double)c->stride * c->n <= 200e6 ? 0.6 : 0.95;
+    const double per_row_us = (double)c->bytes_per_rank * c->n <= 200e6 ? 0.6 : 0.95;
     const double passes = std::ceil(ncols / resident);
     const double column_rate = column_rows <= 128 ? 7.1e6 : column_rows <= 256 ? 6.4e6 : 5.3e6;      // bytes per us
     const double est_column = std::max(bytes / column_rate, (double)column_rows * per_row_us * passes) + 4.0;
@@ -521,8 +526,35 @@ int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
     return SAR_OK;
 }
 
+int sar_adopt_ranks(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
+    if (!c) return set_error(SAR_EINVAL, "context is null");
+    if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
+    if (!device_ptrs) return set_error(SAR_EINVAL, "pointer list is null");
+    if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
+    if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+    SAR_HIP(hipSetDevice(c->device));
+    for (int r = 0; r < n; ++r) {
+        if (!device_ptrs[r]) return set_error(SAR_EINVAL, "a rank pointer is null");
+        if ((uintptr_t)device_ptrs[r] % (uintptr_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "a rank pointer is not aligned to the element size");
+        hipPointerAttribute_t at{};
+        if (hipPointerGetAttributes(&at, device_ptrs[r]) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != c->device) {
+            (void)hipGetLastError();
+            return set_error(SAR_EINVAL, "a rank pointer is not device memory of this context's GPU");
+        }
+        for (int q = 0; q < r; ++q) {
+            const char* a = (const char*)device_ptrs[q]; const char* b = (const char*)device_ptrs[r];
+            if (a < b + bytes_per_rank && b < a + bytes_per_rank) return set_error(SAR_EINVAL, "rank buffers overlap");
+        }
+    }
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    drop_ranks(c);
+    for (int r = 0; r < n; ++r) c->adopted.push_back((char*)device_ptrs[r]);
+    c->n = n; c->dtype = dtype; c->bytes_per_rank = bytes_per_rank; c->stride = 0;
+    return SAR_OK;
+}
+
 static int check_rank_range(sar_ctx* c, int rank, uint64_t off, uint64_t bytes) {
-    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (rank < 0 || rank >= c->n) return set_error(SAR_EINVAL, "rank out of range");
     if (off > c->bytes_per_rank || bytes > c->bytes_per_rank - off) return set_error(SAR_EINVAL, "range leaves the rank buffer");
     return SAR_OK;
@@ -547,7 +579,7 @@ int sar_download(sar_ctx* c, int rank, uint64_t byte_off, void* host, uint64_t b
 }
 
 int sar_fill_const(sar_ctx* c, int rank, uint64_t elem_off, uint64_t elems, double value) {
-    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     const uint64_t es = elem_size_of(c->dtype);
     if (elem_off > c->elems() || elems > c->elems() - elem_off) return set_error(SAR_EINVAL, "range leaves the rank buffer");
     int rc = check_rank_range(c, rank, elem_off * es, elems * es); if (rc) return rc;
@@ -558,7 +590,7 @@ int sar_fill_const(sar_ctx* c, int rank, uint64_t elem_off, uint64_t elems, doub
 }
 
 int sar_fill_reference_pattern(sar_ctx* c, const char* alg, float delay_ms, int base) {
-    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (!alg) return set_error(SAR_EINVAL, "alg is null");
     const std::string a(alg);
     if (a != "stragglar" && a != "ring" && a != "rhd" && a != "direct") return set_error(SAR_EINVAL, "unknown algorithm");
@@ -590,28 +622,39 @@ int sar_fill_uniform(sar_ctx* c, int rank, uint64_t seed, double lo, double hi) 
 int sar_fill_normal(sar_ctx* c, int rank, uint64_t seed, double mean, double std) { return fill_random(c, rank, seed, mean, std, 1); }
 
 int sar_snapshot(sar_ctx* c) {
-    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     SAR_HIP(hipSetDevice(c->device));
-    const uint64_t total = c->stride * (uint64_t)c->n;
+    const uint64_t stride = c->snapshot_stride();
     if (!c->snapshot) {
-        hipError_t e = hipMalloc((void**)&c->snapshot, total);
+        hipError_t e = hipMalloc((void**)&c->snapshot, stride * (uint64_t)c->n);
         if (e != hipSuccess) { (void)hipGetLastError(); c->snapshot = nullptr; return set_error(SAR_ENOMEM, std::string("snapshot: ") + hipGetErrorString(e)); }
     }
-    SAR_HIP(hipMemcpyAsync(c->snapshot, c->arena, total, hipMemcpyDeviceToDevice, c->stream));
+    if (c->adopted.empty()) {
+        SAR_HIP(hipMemcpyAsync(c->snapshot, c->arena, stride * (uint64_t)c->n, hipMemcpyDeviceToDevice, c->stream));
+    } else {
+        for (int r = 0; r < c->n; ++r)
+            SAR_HIP(hipMemcpyAsync(c->snapshot + (uint64_t)r * stride, c->rank_base(r), c->bytes_per_rank, hipMemcpyDeviceToDevice, c->stream));
+    }
     SAR_HIP(hipStreamSynchronize(c->stream));
     return SAR_OK;
 }
 
 int sar_restore(sar_ctx* c) {
-    if (!c || !c->arena || !c->snapshot) return set_error(SAR_ESTATE, "no snapshot taken");
+    if (!c || !c->has_ranks() || !c->snapshot) return set_error(SAR_ESTATE, "no snapshot taken");
     SAR_HIP(hipSetDevice(c->device));
-    SAR_HIP(hipMemcpyAsync(c->arena, c->snapshot, c->stride * (uint64_t)c->n, hipMemcpyDeviceToDevice, c->stream));
+    const uint64_t stride = c->snapshot_stride();
+    if (c->adopted.empty()) {
+        SAR_HIP(hipMemcpyAsync(c->arena, c->snapshot, stride * (uint64_t)c->n, hipMemcpyDeviceToDevice, c->stream));
+    } else {
+        for (int r = 0; r < c->n; ++r)
+            SAR_HIP(hipMemcpyAsync(c->rank_base(r), c->snapshot + (uint64_t)r * stride, c->bytes_per_rank, hipMemcpyDeviceToDevice, c->stream));
+    }
     SAR_HIP(hipStreamSynchronize(c->stream));
     return SAR_OK;
 }
 
 int sar_ranks_identical(sar_ctx* c, uint64_t elems, int* identical) {
-    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (!identical || elems > c->elems()) return set_error(SAR_EINVAL, "bad argument");
     SAR_HIP(hipSetDevice(c->device));
     int zero = 0;
@@ -637,7 +680,7 @@ int sar_set_tuning(sar_ctx* c, const sar_tuning_t* in) {
 }
 
 int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph) {
-    if (!c || !c->arena) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (!main_sched) return set_error(SAR_EINVAL, "main schedule is null");
     for (const sar_schedule* s : {prework, main_sched}) {
         if (!s) continue;
@@ -722,7 +765,10 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     if (!(delay_ms <= kMaxDelayMs)) return set_error(SAR_EINVAL, "delay out of range");
     SAR_HIP(hipSetDevice(c->device));
     SAR_HIP(hipEventRecord(c->ev_start, c->stream));
-    if (delay_ms >= 0) {
+    if (delay_ms == 0) {
+        // nobody is late: pre-work, then the schedule, on one stream
+        int rc = launch_all(c, c->prework); if (rc) return rc;
+    } else if (delay_ms > 0) {
         // the straggler's stream is busy for delay_ms while the others do their pre-work
         const uint64_t ticks = (uint64_t)((double)delay_ms * (double)c->wall_khz);
         SAR_HIP(hipStreamWaitEvent(c->straggler_stream, c->ev_start, 0));
@@ -735,7 +781,7 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     else { int rc = launch_main(c); if (rc) return rc; }
     SAR_HIP(hipEventRecord(c->ev_stop, c->stream));
     SAR_HIP(hipEventSynchronize(c->ev_stop));
-    if (delay_ms >= 0) SAR_HIP(hipStreamSynchronize(c->straggler_stream));
+    if (delay_ms > 0) SAR_HIP(hipStreamSynchronize(c->straggler_stream));
     float ms = 0.f;
     SAR_HIP(hipEventElapsedTime(&ms, c->ev_start, c->ev_stop));
     if (elapsed_ms) *elapsed_ms = ms;

@@ -1,0 +1,125 @@
+"""Single-process emulation of the reference's torch backend on one GPU.
+
+The reference registers a c10d backend ("dummy") whose ``allreduce`` runs the
+8-rank StragglAR schedule with one process and one GPU per rank
+(implementation/custom_backend/src/dummy.cpp: BackendDummy::allreduce :717-729
+-> allreduce_stragglar :256-656: in-place ReduceScatter among the ranks that
+are on time, then the table), and its trainer all-reduces one flat gradient
+buffer per step (implementation/custom_backend/dp.py: flatten_tensors :28,
+allreduce_gradients :50-65: flatten -> all_reduce(SUM) -> divide by the world
+size -> unflatten).
+
+Here all ranks are emulated in ONE process on ONE GPU: the caller hands over
+one tensor per emulated rank and the library works on those tensors in place
+(``sar_adopt_ranks``: no copy into an arena).  torch is used for the tensors
+only; the schedule runs in the HIP library.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional, Sequence
+
+from . import capi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_TORCH_DTYPES = {"torch.float32": "f32", "torch.float16": "f16", "torch.bfloat16": "bf16"}
+
+
+class EmulatedGroup:
+    """n emulated ranks sharing one GPU.
+
+    ``straggler_rank`` names the rank that is late; as in the reference it is
+    relabelled to be the last rank by swapping it with rank n-1
+    (dummy.cpp:157-166, dp.py:71-77).  ``algorithm`` is "stragglar" (default),
+    "ring", "rhd" or "direct".
+    """
+
+    def __init__(self, world_size: int, straggler_rank: Optional[int] = None, algorithm: str = "stragglar",
+                 device: int = 0, schedule_text: Optional[str] = None):
+        if world_size < 3:
+            raise ValueError("world_size must be at least 3")
+        self.n = world_size
+        self.straggler = world_size - 1 if straggler_rank is None else straggler_rank
+        if not 0 <= self.straggler < world_size:
+            raise ValueError("straggler_rank out of range")
+        self.algorithm = algorithm
+        self.device = device
+        self._lib = capi.load_library()
+        self._ctx = self._lib.context(device)
+        if algorithm == "stragglar":
+            if schedule_text is None:
+                path = os.path.join(_HERE, "schedules", "stragglar_n%d.txt" % world_size)
+                if os.path.exists(path):
+                    with open(path) as f:
+                        schedule_text = f.read()
+            self._main = (self._lib.parse(schedule_text, world_size) if schedule_text
+                          else self._lib.builtin("stragglar", world_size))
+            self._prework = self._lib.builtin("prework_rs", world_size)
+        else:
+            self._main = self._lib.builtin(algorithm, world_size)
+            self._prework = self._lib.builtin("prework_ar", world_size) if algorithm == "direct" else None
+        reason = self._main.validate()
+        if reason:
+            raise ValueError("invalid schedule: " + reason)
+        self._key = None
+
+    def close(self):
+        self._ctx.close()
+
+    def _order(self, tensors):
+        """Rank order seen by the schedule: the straggler takes the last place."""
+        order = list(range(self.n))
+        order[self.straggler], order[self.n - 1] = order[self.n - 1], order[self.straggler]
+        return [tensors[i] for i in order]
+
+    def all_reduce(self, tensors: Sequence, delay_ms: float = 0.0) -> float:
+        """Sum-AllReduce in place: ``tensors[r]`` is rank r's flat buffer.  Afterwards every tensor holds the
+        sum.  The element count must divide by world_size-1 for StragglAR (world_size for ring / rhd), as in the
+        reference, whose callers pad their buffers (example.py:19).  ``delay_ms > 0`` makes the straggler late
+        by that much.  Returns the elapsed milliseconds."""
+        import torch
+        if len(tensors) != self.n:
+            raise ValueError("need one tensor per emulated rank")
+        t0 = tensors[0]
+        dtype = _TORCH_DTYPES.get(str(t0.dtype))
+        if dtype is None:
+            raise TypeError("unsupported dtype %s" % t0.dtype)
+        for t in tensors:
+            if not t.is_cuda or t.device.index != self.device or not t.is_contiguous() or t.dtype != t0.dtype or t.numel() != t0.numel():
+                raise ValueError("rank tensors must be contiguous CUDA tensors of one dtype and size on device %d" % self.device)
+        parts = self._main.parts
+        if t0.numel() % parts:
+            raise ValueError("element count %d does not divide into %d chunks: pad the buffer" % (t0.numel(), parts))
+        ordered = self._order(tensors)
+        nbytes = t0.numel() * t0.element_size()
+        key = (tuple(t.data_ptr() for t in ordered), nbytes, dtype)
+        if key != self._key:                       # new buffers: adopt them and lower the schedule onto them
+            self._ctx.adopt_ranks(list(key[0]), nbytes, dtype)
+            self._ctx.prepare(self._main, self._prework)
+            self._key = key
+        torch.cuda.current_stream(self.device).synchronize()     # the caller's pending work on the tensors
+        return self._ctx.run(delay_ms)                            # blocks until the result is complete
+
+    def allreduce_gradients(self, per_rank_grads: Sequence[Sequence], average: bool = True):
+        """dp.py:28-65 for all emulated ranks at once: flatten each rank's gradient tensors into one padded
+        buffer, AllReduce, divide by the world size, copy back into the gradient tensors."""
+        import torch
+        if len(per_rank_grads) != self.n:
+            raise ValueError("need one gradient list per emulated rank")
+        parts = self._main.parts
+        flats = []
+        for grads in per_rank_grads:
+            flat = torch.cat([g.reshape(-1) for g in grads])
+            pad = (-flat.numel()) % parts
+            if pad:
+                flat = torch.cat([flat, flat.new_zeros(pad)])
+            flats.append(flat.contiguous())
+        self.all_reduce(flats)
+        for grads, flat in zip(per_rank_grads, flats):
+            if average:
+                flat.div_(self.n)
+            off = 0
+            for g in grads:
+                g.copy_(flat[off:off + g.numel()].view_as(g))
+                off += g.numel()
+        return flats

@@ -74,7 +74,7 @@ def test_parity_small(gpu_ctx, sarlib, oracle, n, alg, dtype, executor):
 
 
 def test_config1_n4_1mib_fp32(gpu_ctx, sarlib, oracle):
-    """BASELINE config 1: n=4 StragglAR, 1 MiB fp32 per rank (padded: 1 050 624 B), uniform[-1,1) seed 0,
+    """Benchmark configuration 1 (the reference's own CPU-runnable case): n=4 StragglAR, 1 MiB fp32 per rank (padded: 1 050 624 B), uniform[-1,1) seed 0,
     pre-work materialised by the ReduceScatter, then the table with delay -1 semantics."""
     n, dtype = 4, "f32"
     nbytes = sarlib.pad_bytes(1 << 20, n)
@@ -100,7 +100,7 @@ def shipped_table(n):
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 def test_config4_shape_n6_nonpow2_with_prework(gpu_ctx, sarlib, oracle, dtype):
-    """BASELINE config 4 at a size the checker finishes quickly: n=6 table from the non-power-of-two
+    """Benchmark configuration 4 at a size the checker finishes quickly: n=6 table from the non-power-of-two
     synthesizer, fp16 uniform[-0.5,0.5), padded per pad_buffers.py, ReduceScatter pre-work on ranks 0-4."""
     n = 6
     nbytes = sarlib.pad_bytes(1 << 20, n)
@@ -350,7 +350,7 @@ def gather_slices(ctx, rank, chunk, parts, offs, length):
 
 @pytest.mark.parametrize("executor", [0, 1])
 def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
-    """BASELINE config 2 at its real size: n=8, 256 MiB fp32 per rank (2 GiB resident), uniform[-1,1)
+    """Benchmark configuration 2 (the one the headline figure is quoted on) at its real size: n=8, 256 MiB fp32 per rank (2 GiB resident), uniform[-1,1)
     seeded per rank, stragglar (both tables) / ring / rhd / direct on the same inputs.  Every op is
     element-wise within chunk structure, so parity is checked on a mini problem gathered from the
     same positions of every chunk, plus `all ranks identical` over the whole buffers."""
@@ -390,7 +390,7 @@ def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
 
 
 def test_config3_bf16_1gib_with_delay(gpu_ctx, sarlib, oracle):
-    """BASELINE config 3: n=8 x 1 GiB bf16 (padded 1 073 744 896 B), normal(0, 1e-3) seeded per rank,
+    """Benchmark configuration 3: n=8 x 1 GiB bf16 (padded 1 073 744 896 B), normal(0, 1e-3) seeded per rank,
     sums accumulated in bf16, straggler rank 7 late by DELAY = 5 ms while ranks 0-6 reduce-scatter."""
     n, dtype = 8, "bf16"
     nbytes = sarlib.pad_bytes(1 << 30, n)
@@ -417,7 +417,7 @@ def test_config3_bf16_1gib_with_delay(gpu_ctx, sarlib, oracle):
 
 
 def test_config4_full_size_n6_fp16(gpu_ctx, sarlib, oracle):
-    """BASELINE config 4: n=6 x 64 MiB fp16 (padded 67 112 960 B), uniform[-0.5,0.5), pre-work on ranks 0-4,
+    """Benchmark configuration 4: n=6 x 64 MiB fp16 (padded 67 112 960 B), uniform[-0.5,0.5), pre-work on ranks 0-4,
     against the checker on the whole buffers."""
     n, dtype = 6, "f16"
     nbytes = sarlib.pad_bytes(64 << 20, n)
@@ -440,8 +440,8 @@ def test_config4_full_size_n6_fp16(gpu_ctx, sarlib, oracle):
 
 @pytest.mark.parametrize("nbytes", [4 << 10, 64 << 10, 1 << 20, 16 << 20])
 def test_config5_message_size_sweep(gpu_ctx, sarlib, oracle, nbytes):
-    """BASELINE config 5 (the sizes the checker handles on whole buffers; 256 MiB and 1 GiB are covered
-    by the config 2 and 3 tests): n=8 fp32, four algorithms, graph on and off."""
+    """Benchmark configuration 5, the message-size sweep (the sizes the checker handles on whole buffers; 256 MiB and 1 GiB are covered
+    by the tests of configurations 2 and 3): n=8 fp32, four algorithms, graph on and off."""
     n, dtype = 8, "f32"
     padded = sarlib.pad_bytes(nbytes, n)
     inputs = make_inputs(n, padded // 4, dtype, seed=nbytes % 1000)

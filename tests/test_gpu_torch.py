@@ -1,0 +1,113 @@
+"""The single-process torch front end (one tensor per emulated rank, worked on in place through
+sar_adopt_ranks) against the CPU checker and against torch's own sum."""
+import numpy as np
+import pytest
+
+from conftest import assert_bits_equal, read_golden
+from oracle import parse_table
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def rank_tensors(n, numel, dtype, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return [(torch.rand(numel, generator=g, dtype=torch.float32) * 2 - 1).to(dtype).cuda() for _ in range(n)]
+
+
+def to_np_bits(t):
+    if t.dtype == torch.float32:
+        return t.cpu().numpy()
+    return t.cpu().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.float32, "f32"), (torch.bfloat16, "bf16"), (torch.float16, "f16")])
+def test_all_reduce_in_place_matches_checker(oracle, dtype, name):
+    from stragglar_amd.torch_emulation import EmulatedGroup
+    n, numel = 8, 7 * 8 * 4096 + 7 * 8
+    tensors = rank_tensors(n, numel, dtype, seed=1)
+    inputs = [to_np_bits(t).copy() for t in tensors]
+    ptrs = [t.data_ptr() for t in tensors]
+    group = EmulatedGroup(n)
+    try:
+        ms = group.all_reduce(tensors)
+        assert ms > 0
+        assert [t.data_ptr() for t in tensors] == ptrs                      # in place, nothing reallocated
+        want = [x.copy() for x in inputs]
+        oracle.run("stragglar", want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+        for r in range(n):
+            assert_bits_equal(to_np_bits(tensors[r]), want[r], "rank %d" % r)
+        # a second call on the same tensors reuses the lowered plan and sums the sums
+        group.all_reduce(tensors)
+        oracle.run("stragglar", want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+        for r in range(n):
+            assert_bits_equal(to_np_bits(tensors[r]), want[r], "second call, rank %d" % r)
+    finally:
+        group.close()
+
+
+def test_straggler_relabelling_and_comparators(oracle):
+    """STRAGGLER_RANK = 6 in the reference (dummy.cpp:157, dp.py:22): whichever rank is late, every rank ends
+    with the same sum; the relabelled order decides the association, which the checker reproduces."""
+    from stragglar_amd.torch_emulation import EmulatedGroup
+    n, numel = 8, 7 * 8 * 1024
+    for alg in ("stragglar", "ring", "rhd", "direct"):
+        tensors = rank_tensors(n, numel, torch.float32, seed=2)
+        inputs = [t.cpu().numpy().copy() for t in tensors]
+        group = EmulatedGroup(n, straggler_rank=6, algorithm=alg)
+        try:
+            group.all_reduce(tensors)
+        finally:
+            group.close()
+        order = list(range(n))
+        order[6], order[7] = order[7], order[6]
+        want = [inputs[i].copy() for i in order]
+        oracle.run(alg, want, "f32", rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+        for k, i in enumerate(order):
+            assert_bits_equal(tensors[i].cpu().numpy(), want[k], "%s rank %d" % (alg, i))
+        total = np.sum(np.stack(inputs).astype(np.float64), axis=0)
+        assert np.allclose(tensors[0].cpu().numpy(), total, rtol=0, atol=1e-5)
+
+
+def test_gradient_averaging_like_the_reference_trainer():
+    """dp.py:28-65: flatten -> all_reduce(SUM) -> / world_size -> unflatten, for all emulated ranks."""
+    from stragglar_amd.torch_emulation import EmulatedGroup
+    n = 4
+    shapes = [(33, 7), (129,), (5, 5, 5)]
+    g = torch.Generator(device="cpu").manual_seed(3)
+    grads = [[torch.randn(s, generator=g).cuda() for s in shapes] for _ in range(n)]
+    expect = [sum(grads[r][k].double() for r in range(n)) / n for k in range(len(shapes))]
+    group = EmulatedGroup(n)
+    try:
+        group.allreduce_gradients(grads)
+    finally:
+        group.close()
+    for r in range(n):
+        for k in range(len(shapes)):
+            assert torch.allclose(grads[r][k].double(), expect[k], rtol=0, atol=1e-6)
+
+
+def test_adopt_rejects_bad_buffers(sarlib):
+    import stragglar_amd as sa
+    ctx = sarlib.context(0)
+    try:
+        t = torch.zeros(1024, device="cuda")
+        with pytest.raises(sa.SarError):
+            ctx.adopt_ranks([t.data_ptr(), t.data_ptr() + 1024], 4096, "f32")        # overlapping
+        with pytest.raises(sa.SarError):
+            ctx.adopt_ranks([t.data_ptr(), 0], 1024, "f32")                          # null
+        host = np.zeros(1024, np.float32)
+        with pytest.raises(sa.SarError):
+            ctx.adopt_ranks([t.data_ptr(), host.ctypes.data], 1024, "f32")           # host memory
+        ctx.adopt_ranks([t.data_ptr(), t.data_ptr() + 2048], 2048, "f32")
+        ctx.fill_const(0, 2.0)
+        ctx.fill_const(1, 3.0)
+        ctx.snapshot()
+        ctx.prepare(sarlib.builtin("ring", 2))
+        ctx.run(-1.0)
+        assert torch.all(t == 5.0)
+        ctx.restore()
+        assert torch.all(t[:512] == 2.0) and torch.all(t[512:] == 3.0)
+    finally:
+        ctx.close()
