@@ -126,6 +126,14 @@ def main():
     wall_s = time.perf_counter() - t_wall0
     identical = ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts)
     ms = statistics.fmean(step_ms)
+    # the same K steps back to back on the host clock, no restore in between (the sums just keep growing):
+    # a cross-check of the event timing that includes launch and synchronisation overhead
+    ctx.restore()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ctx.run(-1.0)
+    back_to_back_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ctx.restore()
     value = st.algorithmic_bytes / ms / 1e6
 
     # per-launch durations of the dominant kernel (sar::round_kernel), events on the launch stream
@@ -164,6 +172,7 @@ def main():
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
         "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),
+        "wall_ms_per_step_back_to_back": round(back_to_back_ms, 4),
         "ranks_identical_after_run": bool(identical),
         "roofline": roofline,
     }

@@ -77,6 +77,10 @@ typedef struct sar_stats_t {
     int32_t uses_graph;            /* 1 if sar_run replays a hipGraph                                             */
     int32_t executor;              /* executor the main schedule was lowered for: 0 per round, 1 column           */
     int32_t col_block;             /* column executor: threads per workgroup in use (0 otherwise)                 */
+    int32_t col_slots;             /* column executor: value slots per lane in use (0 = no forwarding)            */
+    int32_t reserved;
+    uint64_t forwarded_bytes;      /* part of algorithmic_bytes that the column executor takes from value slots   */
+                                   /* in LDS instead of loading it again from the rank buffers                    */
 } sar_stats_t;
 
 /* run-time tunables of the round kernel; sar_get_tuning() reports the defaults */
@@ -98,6 +102,13 @@ typedef struct sar_tuning_t {
     int32_t col_wgs;      /* column executor: workgroups per compute unit in the grid                */
     int32_t col_block;    /* column executor: threads per workgroup = 16-byte vectors per column     */
                           /*     (256, 512 or 1024; 0 = chosen from the number of columns)           */
+    int32_t col_forward;  /* column executor: 1 = a value a lane wrote in an earlier round and needs  */
+                          /*     again is kept in LDS and not loaded again (all stores still happen; */
+                          /*     same bits); 0 = every operand is loaded from its rank buffer        */
+    int32_t col_slots;    /* column executor: most values kept per lane (0 = as many as fit in LDS)  */
+    int32_t col_light_sync; /* column executor: 1 = between rounds the waves of a workgroup only meet   */
+                          /*     (no wait for their stores) whenever no lane reads bytes another lane */
+                          /*     wrote; 0 = always a full barrier                                     */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1};
 
     // prepared plan
     bool prepared = false;
@@ -69,7 +69,7 @@ struct sar_ctx {
     // column plan (tune.executor == 1): the whole main schedule as one launch
     bool column = false;
     uint32_t* d_round_begin = nullptr;
-    uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512;
+    uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512, col_slots = 0, col_lane_local = 0;
     int cu_count = 0;
 
     std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
@@ -88,7 +88,7 @@ void drop_plan(sar_ctx* c) {
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
     if (c->d_round_begin) { (void)hipFree(c->d_round_begin); c->d_round_begin = nullptr; }
-    c->column = false; c->col_rounds = c->col_count = c->col_grid = 0;
+    c->column = false; c->col_rounds = c->col_count = c->col_grid = c->col_slots = 0;
     c->prework.clear(); c->rounds.clear(); c->prepared = false;
     c->stats = sar_stats_t{};
 }
@@ -281,86 +281,246 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
 
 // Column plan: every row of the main schedule, cut into single-chunk rows (all rows then share one
 // within-chunk offset space), in round order, plus the index of each round's first row.
-int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std::vector<uint32_t>& round_begin, uint64_t* widest_row) {
+//
+// Value forwarding.  A lane of the column kernel meets the same (rank, chunk) cells again and again: what
+// round r writes, later rounds read back.  The kernel can keep up to `nslots` such values per lane in LDS
+// (write-through: every value is stored to its rank buffer as well), and which read finds its operand
+// there is decided here, on the host, by running the slot bookkeeping over the rows once: a slot stands
+// for one value and the set of cells that currently equal it (a COPY from a held value adds its
+// destination to the set at no cost; a write to a cell takes it out of its old set).  When all slots
+// are busy the value whose next use is furthest away gives way, which is known exactly because the
+// whole schedule is.  Rows get DEVOP_GET0 / GET1 / PUT and their slot numbers; the cache policy is
+// then planned on the reads that still go to memory.
+struct ColumnPlan {
+    std::vector<uint32_t> round_begin;
+    uint64_t widest_row = 0;
+    int block = 512;
+    uint32_t nslots = 0;
+    uint64_t forwarded_bytes = 0;    // operand bytes taken from value slots instead of memory, per run
+    bool lane_local = false;         // every row 16-byte aligned and a whole number of vectors long
+};
+
+int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, ColumnPlan& plan) {
     const int es = elem_size_of(c->dtype);
     const uint64_t elems = c->elems();
     const uint64_t chunk_bytes = (elems / (uint64_t)s.parts) * es;
-    std::vector<std::vector<RowAccess>> acc;
-    for (const auto& round : s.rounds) {
-        std::vector<RowAccess> v;
-        for (const auto& op : round) v.push_back(accesses(s, op, elems, es));
-        acc.push_back(v);
-    }
-    // a column keeps its data close for the whole schedule: anything read again in ANY later round stays cached
-    auto read_later = [&](size_t round, const Touch& t) {
-        for (size_t r = round + 1; r < acc.size(); ++r)
-            for (const auto& ra : acc[r])
-                for (const auto& rd : ra.reads)
-                    if (overlaps(rd, t)) return true;
-        return false;
+    const int cells_per_rank = s.parts + 1;
+    auto cell_of = [&](int rank, uint64_t byte_off) {
+        return rank * cells_per_rank + (int)(chunk_bytes ? std::min<uint64_t>(byte_off / chunk_bytes, (uint64_t)s.parts) : 0);
     };
-    *widest_row = 0;
-    const size_t first = rows.size();          // round_begin counts from the first column row
+    struct ColRow { sar::DevOp d; int c0, c1; };
+    std::vector<ColRow> cr;
+    plan.round_begin.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0;
     for (size_t ri = 0; ri < s.rounds.size(); ++ri) {
-        round_begin.push_back((uint32_t)(rows.size() - first));
-        for (size_t oi = 0; oi < s.rounds[ri].size(); ++oi) {
-            const sar::Op& op = s.rounds[ri][oi];
+        plan.round_begin.push_back((uint32_t)cr.size());
+        for (const sar::Op& op : s.rounds[ri]) {
             if (op.kind == SAR_OP_MREDUCE) return set_error(SAR_ESCHED, "internal: multi-source rows have no column form");
             sar::Range rg = sar::lower_range(s, op, elems);
             const uint64_t row_bytes = rg.len * es;
             if (row_bytes == 0) continue;
             const uint64_t row_doff = rg.dst_off * es, row_soff = rg.src_off * es;
             if (row_doff + row_bytes > c->bytes_per_rank || row_soff + row_bytes > c->bytes_per_rank) return set_error(SAR_ESCHED, "row leaves the rank buffer");
-            uint32_t flags = 0;
-            const RowAccess& ra = acc[ri][oi];
-            if (c->tune.cache_policy == 1) {
-                flags = sar::DEVOP_LNT | sar::DEVOP_SNT0 | sar::DEVOP_SNT1;
-            } else if (c->tune.cache_policy == 2) {
-                bool again = false;
-                for (const auto& rd : ra.reads) again |= read_later(ri, rd);
-                if (!again) flags |= sar::DEVOP_LNT;
-                if (!read_later(ri, ra.writes[0])) flags |= sar::DEVOP_SNT0;
-                if (ra.writes.size() > 1 && !read_later(ri, ra.writes[1])) flags |= sar::DEVOP_SNT1;
-            }
             for (int j = 0; j < op.nchunks; ++j) {
                 const uint64_t base = (uint64_t)j * chunk_bytes;
-                sar::DevOp d{};
-                d.kind = (uint32_t)op.kind;
-                d.bytes = (j == op.nchunks - 1) ? row_bytes - base : chunk_bytes;     // a to_end row ends with a longer chunk
-                d.p0 = c->rank_base(op.dst_rank) + row_doff + base;
-                d.p1 = c->rank_base(op.src_rank) + row_soff + base;
-                d.flags = flags | (((((uintptr_t)d.p0 | (uintptr_t)d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u);
-                *widest_row = std::max(*widest_row, d.bytes);
-                rows.push_back(d);
+                ColRow r{};
+                r.d.kind = (uint32_t)op.kind;
+                r.d.bytes = (j == op.nchunks - 1) ? row_bytes - base : chunk_bytes;     // a to_end row ends with a longer chunk
+                r.d.p0 = c->rank_base(op.dst_rank) + row_doff + base;
+                r.d.p1 = c->rank_base(op.src_rank) + row_soff + base;
+                r.d.flags = ((((uintptr_t)r.d.p0 | (uintptr_t)r.d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u;
+                r.c0 = cell_of(op.dst_rank, row_doff + base);
+                r.c1 = cell_of(op.src_rank, row_soff + base);
+                plan.widest_row = std::max(plan.widest_row, r.d.bytes);
+                cr.push_back(r);
             }
         }
     }
-    round_begin.push_back((uint32_t)(rows.size() - first));
+    plan.round_begin.push_back((uint32_t)cr.size());
+    if (cr.size() > 0x7ffffff0ull) return set_error(SAR_EINVAL, "schedule has too many rows");
+    const uint32_t nrows = (uint32_t)cr.size();
+    const uint32_t never = 0xffffffffu;
+
+    // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
+    plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512) >= 2048 ? 512 : 256);
+    // per cell, the rows that touch it, in order; a reducing row reads and writes its cell
+    const int ncells = c->n * cells_per_rank;
+    struct Ev { uint32_t row; bool reads, writes; };
+    std::vector<std::vector<Ev>> ev((size_t)ncells);
+    for (uint32_t i = 0; i < nrows; ++i) {
+        const bool reduce = cr[i].d.kind != SAR_OP_COPY, both = cr[i].d.kind == SAR_OP_XREDUCE;
+        ev[(size_t)cr[i].c0].push_back({i, reduce, true});
+        if (cr[i].c1 != cr[i].c0) ev[(size_t)cr[i].c1].push_back({i, true, both});
+    }
+    // the next row after `i` that reads the cell's present value (never: it is overwritten first, or not read again)
+    auto next_read = [&](int cell, uint32_t i) {
+        const auto& v = ev[(size_t)cell];
+        auto it = std::upper_bound(v.begin(), v.end(), i, [](uint32_t x, const Ev& e) { return x < e.row; });
+        return (it != v.end() && it->reads) ? it->row : never;
+    };
+
+    // one pass of the slot bookkeeping with at most `max_slots` slots
+    struct Forwarding {
+        std::vector<uint32_t> flags, slots;      // per row: DEVOP_GET0 | GET1 | PUT and the packed slot numbers
+        uint32_t nslots = 0;
+        uint64_t bytes = 0;                      // operand bytes found in slots
+    };
+    auto forward = [&](uint32_t max_slots) {
+        Forwarding f;
+        f.flags.assign(nrows, 0); f.slots.assign(nrows, 0);
+        if (max_slots == 0) return f;
+        struct Slot { std::vector<int> cells; uint64_t bytes = 0; };
+        std::vector<Slot> slot(max_slots);
+        std::vector<int> cell_slot((size_t)ncells, -1);
+        auto drop_cell = [&](int cell) {
+            const int k = cell_slot[(size_t)cell];
+            if (k < 0) return;
+            auto& v = slot[(size_t)k].cells;
+            v.erase(std::remove(v.begin(), v.end(), cell), v.end());
+            cell_slot[(size_t)cell] = -1;
+        };
+        auto clear_slot = [&](int k) {
+            for (int cell : slot[(size_t)k].cells) cell_slot[(size_t)cell] = -1;
+            slot[(size_t)k].cells.clear();
+        };
+        auto slot_next_use = [&](int k, uint32_t i) {
+            uint32_t m = never;
+            for (int cell : slot[(size_t)k].cells) m = std::min(m, next_read(cell, i));
+            return m;
+        };
+        // a slot for a value next used at row `nu`: a free one, else the one whose own next use is furthest (and later than nu)
+        auto take_slot = [&](uint32_t nu, uint32_t i) {
+            int far = -1; uint32_t far_use = 0;
+            for (int k = 0; k < (int)max_slots; ++k) {
+                if (slot[(size_t)k].cells.empty()) return k;
+                const uint32_t u = slot_next_use(k, i);
+                if (u == never) { clear_slot(k); return k; }
+                if (u > far_use) { far_use = u; far = k; }
+            }
+            if (far >= 0 && far_use > nu) { clear_slot(far); return far; }
+            return -1;
+        };
+        for (uint32_t i = 0; i < nrows; ++i) {
+            const sar::DevOp& d = cr[i].d;
+            const int c0 = cr[i].c0, c1 = cr[i].c1;
+            const bool reduce = d.kind != SAR_OP_COPY;
+            const bool can = (d.flags & sar::DEVOP_VEC) && c0 != c1;
+            int k0 = (can && reduce) ? cell_slot[(size_t)c0] : -1, k1 = can ? cell_slot[(size_t)c1] : -1;
+            if (k0 >= 0 && slot[(size_t)k0].bytes != d.bytes) k0 = -1;
+            if (k1 >= 0 && slot[(size_t)k1].bytes != d.bytes) k1 = -1;
+            if (k0 >= 0) { f.flags[i] |= sar::DEVOP_GET0; f.slots[i] |= (uint32_t)k0; f.bytes += d.bytes & ~(uint64_t)15u; f.nslots = std::max(f.nslots, (uint32_t)k0 + 1); }
+            if (k1 >= 0) { f.flags[i] |= sar::DEVOP_GET1; f.slots[i] |= (uint32_t)k1 << 8; f.bytes += d.bytes & ~(uint64_t)15u; f.nslots = std::max(f.nslots, (uint32_t)k1 + 1); }
+            // the row's result replaces what its destination cells held
+            drop_cell(c0);
+            if (d.kind == SAR_OP_XREDUCE) drop_cell(c1);
+            if (d.kind == SAR_OP_COPY && k1 >= 0) {
+                slot[(size_t)k1].cells.push_back(c0); cell_slot[(size_t)c0] = k1;          // the held value now lives in c0 too
+            } else if (can) {
+                uint32_t nu = next_read(c0, i);
+                if (d.kind != SAR_OP_REDUCE_INTO) nu = std::min(nu, next_read(c1, i));      // COPY: source and destination hold the value
+                const int k = nu == never ? -1 : take_slot(nu, i);
+                if (k >= 0) {
+                    if (d.kind == SAR_OP_COPY) drop_cell(c1);
+                    slot[(size_t)k].bytes = d.bytes;
+                    slot[(size_t)k].cells.push_back(c0); cell_slot[(size_t)c0] = k;
+                    if (d.kind != SAR_OP_REDUCE_INTO) { slot[(size_t)k].cells.push_back(c1); cell_slot[(size_t)c1] = k; }
+                    f.flags[i] |= sar::DEVOP_PUT; f.slots[i] |= (uint32_t)k << 16;
+                    f.nslots = std::max(f.nslots, (uint32_t)k + 1);
+                }
+            }
+        }
+        if (f.bytes == 0) { f.flags.assign(nrows, 0); f.slots.assign(nrows, 0); f.nslots = 0; }    // nothing found: no slots at all
+        return f;
+    };
+
+    // How many slots.  LDS per compute unit is what they cost: up to 5 per lane all 2048 lanes of a compute unit
+    // stay resident, up to 10 half of them.  Measured on MI355X, half occupancy pays when every re-read is then
+    // found in a slot (what still goes to memory is the cold inputs and the stores), but not for a part of them;
+    // and a plan that finds less than a tenth of the bytes the rows move is not worth the longer row loop.
+    Forwarding fwd;
+    if (c->tune.col_forward) {
+        const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, sar::column_lds_budget() / sar::column_bytes(plan.block));
+        if (c->tune.col_slots > 0) {
+            fwd = forward(std::min<uint32_t>(fit, (uint32_t)c->tune.col_slots));
+        } else {
+            const uint64_t all = forward(255u).bytes;
+            fwd = forward(std::min<uint32_t>(fit, 10u));
+            if (fwd.bytes != all) fwd = forward(std::min<uint32_t>(fit, 5u));
+            uint64_t moved = 0;                  // algorithmic bytes of the rows
+            for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : 3u);
+            if (fwd.bytes * 10u < moved) fwd = forward(0);
+        }
+    } else {
+        fwd = forward(0);
+    }
+    plan.nslots = fwd.nslots; plan.forwarded_bytes = fwd.bytes;
+    std::vector<uint8_t> memread0(nrows, 0), memread1(nrows, 0);
+    for (uint32_t i = 0; i < nrows; ++i) {
+        cr[i].d.flags |= fwd.flags[i]; cr[i].d.slots = fwd.slots[i];
+        memread0[i] = cr[i].d.kind != SAR_OP_COPY && !(fwd.flags[i] & sar::DEVOP_GET0);
+        memread1[i] = !(fwd.flags[i] & sar::DEVOP_GET1);
+    }
+
+    // Cache policy over the accesses that go to memory.  Without forwarding a column keeps its data close for the
+    // whole schedule: anything read again in ANY later row stays cached.  With forwarding what is left is mostly
+    // read or written once, and streaming everything measured faster also for the re-reads that found no slot.
+    if (c->tune.cache_policy == 1 || (c->tune.cache_policy == 2 && plan.nslots > 0)) {
+        for (auto& r : cr) r.d.flags |= sar::DEVOP_LNT | sar::DEVOP_SNT0 | sar::DEVOP_SNT1;
+    } else if (c->tune.cache_policy == 2) {
+        std::vector<uint8_t> read_later((size_t)ncells, 0);
+        // rows of one round neither read what another row of the round writes, so "later" may go row by row
+        for (uint32_t i = nrows; i-- > 0;) {
+            sar::DevOp& d = cr[i].d;
+            const int c0 = cr[i].c0, c1 = cr[i].c1;
+            bool again = false;
+            if (memread0[i]) again |= read_later[(size_t)c0] != 0;
+            if (memread1[i]) again |= read_later[(size_t)c1] != 0;
+            if (!again) d.flags |= sar::DEVOP_LNT;
+            if (!read_later[(size_t)c0]) d.flags |= sar::DEVOP_SNT0;
+            if (d.kind == SAR_OP_XREDUCE && !read_later[(size_t)c1]) d.flags |= sar::DEVOP_SNT1;
+            if (memread0[i]) read_later[(size_t)c0] = 1;
+            if (memread1[i]) read_later[(size_t)c1] = 1;
+        }
+    }
+    plan.lane_local = true;
+    for (const auto& r : cr) {
+        if (!(r.d.flags & sar::DEVOP_VEC) || (r.d.bytes & 15u)) plan.lane_local = false;
+        rows.push_back(r.d);
+    }
     return SAR_OK;
 }
 
-// Which executor is expected to be faster (executor = 2).  Constants are measurements on MI355X:
-// the column kernel moves 7.1 algorithmic TB/s when there are columns enough to fill the chip and a
-// column is up to ~128 rows long (n = 8), less for longer columns, whose workgroups drift apart and
-// scatter the access streams (6.4 up to 256 rows, 5.3 beyond); a workgroup needs about 0.6 us per row
-// while everything stays cache resident, 0.95 us beyond that; one launch per round moves 6.5 TB/s and
-// costs about 3 us per launch.
-bool column_pays(const sar_ctx* c, size_t column_rows, uint64_t widest_row, int col_block) {
+// Which executor is expected to be faster (executor = 2).  Constants are measurements on MI355X.
+// Column kernel without forwarding: 7.1 algorithmic TB/s when there are columns enough to fill the chip
+// and a column is up to ~128 rows long (n = 8), less for longer columns, whose workgroups drift apart
+// and scatter the access streams (6.4 up to 256 rows, 5.3 beyond).  With forwarding what counts is the
+// bytes that still go to memory: 5.0 TB/s when they are mostly stores (three tenths or more of the
+// operands found in slots), 6.0 otherwise.  A workgroup needs about 0.6 us per row while everything
+// stays cache resident, 0.95 us beyond that; one launch per round moves 6.5 TB/s and costs about 3 us
+// per launch.
+bool column_pays(const sar_ctx* c, size_t column_rows, const ColumnPlan& cp) {
     const double bytes = (double)c->stats.algorithmic_bytes;
-    const uint64_t cb = sar::column_bytes(col_block);
-    const double ncols = (double)((widest_row + cb - 1) / cb);
-    const double resident = (double)std::max(1, c->cu_count) * (2048.0 / col_block);
+    const uint64_t cb = sar::column_bytes(cp.block);
+    const double ncols = (double)((cp.widest_row + cb - 1) / cb);
+    double wgs_per_cu = 2048.0 / cp.block;
+    if (cp.nslots) wgs_per_cu = std::max(1.0, std::min(wgs_per_cu, std::floor(160.0 * 1024.0 / ((double)cp.nslots * (double)cb))));
+    const double resident = (double)std::max(1, c->cu_count) * wgs_per_cu;
     const double per_row_us = (double)c->bytes_per_rank * c->n <= 200e6 ? 0.6 : 0.95;
     const double passes = std::ceil(ncols / resident);
-    const double column_rate = column_rows <= 128 ? 7.1e6 : column_rows <= 256 ? 6.4e6 : 5.3e6;      // bytes per us
-    const double est_column = std::max(bytes / column_rate, (double)column_rows * per_row_us * passes) + 4.0;
+    double est_stream;
+    if (cp.nslots) {
+        const double to_memory = std::max(0.0, bytes - (double)cp.forwarded_bytes);
+        est_stream = to_memory / ((double)cp.forwarded_bytes >= 0.3 * bytes ? 5.0e6 : 6.0e6);             // bytes per us
+    } else {
+        est_stream = bytes / (column_rows <= 128 ? 7.1e6 : column_rows <= 256 ? 6.4e6 : 5.3e6);
+    }
+    const double est_column = std::max(est_stream, (double)column_rows * per_row_us * passes) + 4.0;
     double est_rounds = 0;
     for (const auto& L : c->rounds) if (L.total_tiles) est_rounds += 3.0 + (double)L.algorithmic_bytes / 6.5e6;
     return est_column <= est_rounds;
 }
 
 int launch_column_once(sar_ctx* c) {
-    SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->stream, c->d_ops + c->col_first_op, c->d_round_begin, c->col_rounds, c->col_count));
+    SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->col_slots, c->col_lane_local, c->stream, c->d_ops + c->col_first_op, c->d_round_begin, c->col_rounds, c->col_count));
     return SAR_OK;
 }
 
@@ -387,7 +547,9 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
            (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256 &&
            (t.executor >= 0 && t.executor <= 2) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
-           (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024);
+           (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024) &&
+           (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
+           (t.col_light_sync == 0 || t.col_light_sync == 1);
 }
 
 }  // namespace
@@ -692,7 +854,7 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_plan(c);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    std::vector<uint32_t> round_begin; uint32_t col_first = 0; uint64_t widest_row = 0; bool want_column = false; int col_block = 512;
+    ColumnPlan cp; uint32_t col_first = 0; bool want_column = false;
     int rc;
     try {
         if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) { drop_plan(c); return rc; }
@@ -702,14 +864,10 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
         for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
         if (columnar) {
             col_first = (uint32_t)rows.size();
-            if ((rc = lower_column(c, main_sched->s, rows, round_begin, &widest_row)) != SAR_OK) { drop_plan(c); return rc; }
+            if ((rc = lower_column(c, main_sched->s, rows, cp)) != SAR_OK) { drop_plan(c); return rc; }
             columnar = rows.size() > col_first;
         }
-        if (columnar) {
-            // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
-            col_block = c->tune.col_block ? c->tune.col_block : (widest_row / sar::column_bytes(512) >= 2048 ? 512 : 256);
-            if (c->tune.executor == 2) columnar = column_pays(c, rows.size() - col_first, widest_row, col_block);
-        }
+        if (columnar && c->tune.executor == 2) columnar = column_pays(c, rows.size() - col_first, cp);
         want_column = columnar;
     } catch (const std::bad_alloc&) { drop_plan(c); return set_error(SAR_ENOMEM, "out of host memory"); }
     if (!rows.empty()) {
@@ -720,13 +878,15 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     if (!ptrs.empty()) SAR_HIP(hipMemcpy(c->d_ptrs, ptrs.data(), ptrs.size() * sizeof(char*), hipMemcpyHostToDevice));
 
     if (want_column) {
-        SAR_HIP(hipMalloc((void**)&c->d_round_begin, round_begin.size() * sizeof(uint32_t)));
-        SAR_HIP(hipMemcpy(c->d_round_begin, round_begin.data(), round_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
-        c->col_block = (uint32_t)col_block;
-        const uint64_t cb = sar::column_bytes(c->col_block);
-        const uint64_t ncols = (widest_row + cb - 1) / cb;
+        SAR_HIP(hipMalloc((void**)&c->d_round_begin, cp.round_begin.size() * sizeof(uint32_t)));
+        SAR_HIP(hipMemcpy(c->d_round_begin, cp.round_begin.data(), cp.round_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        c->col_block = (uint32_t)cp.block;
+        c->col_slots = cp.nslots;
+        c->col_lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
+        const uint64_t cb = sar::column_bytes(cp.block);
+        const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
         if (ncols > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 columns"); }
-        c->col_first_op = col_first; c->col_rounds = (uint32_t)round_begin.size() - 1; c->col_count = (uint32_t)ncols;
+        c->col_first_op = col_first; c->col_rounds = (uint32_t)cp.round_begin.size() - 1; c->col_count = (uint32_t)ncols;
         const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
         c->col_grid = (uint32_t)std::min<uint64_t>(ncols, resident);
         c->column = true;
@@ -755,6 +915,8 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     }
     st.executor = c->column ? 1 : 0;
     st.col_block = c->column ? (int32_t)c->col_block : 0;
+    st.col_slots = c->column ? (int32_t)c->col_slots : 0;
+    st.forwarded_bytes = c->column ? cp.forwarded_bytes : 0;
     c->stats = st;
     c->prepared = true;
     return SAR_OK;

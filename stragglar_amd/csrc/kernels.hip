@@ -349,11 +349,15 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // One row at a time and one vector per lane turned out best (28 VGPRs, eight waves per SIMD resident:
 // the other workgroups of the compute unit cover a row's latency; batching the loads of several rows or
 // several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
-template <int DT, int BLOCK>
+template <int DT, int BLOCK, bool FWD>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ round_begin,
-                                                        uint32_t nrounds, uint32_t ncols) {
+                                                        uint32_t nrounds, uint32_t ncols, uint32_t lane_local) {
     typedef typename Elem<DT>::T T;
     constexpr uint64_t col_bytes = (uint64_t)BLOCK * 16u;
+    // FWD: value slots in LDS, slot k of lane t at vector k*BLOCK + t.  A lane only ever touches its
+    // own vectors, so the slots need no synchronisation of their own.
+    extern __shared__ __align__(16) char lds_raw[];
+    f4* const mine = reinterpret_cast<f4*>(lds_raw) + threadIdx.x;
     for (uint32_t col = blockIdx.x; col < ncols; col += gridDim.x) {
         const uint64_t off = (uint64_t)col * col_bytes;
         const uint64_t voff = off + ((uint64_t)threadIdx.x << 4);       // this lane's vector within every row
@@ -367,13 +371,19 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                 if (flags & DEVOP_VEC) {
                     if (voff + 16u <= bytes) {
                         f4 a = {0.f, 0.f, 0.f, 0.f}, b;
-                        if (flags & DEVOP_LNT) { b = ld16<true>(p1 + voff); if (kind != SAR_OP_COPY) a = ld16<true>(p0 + voff); }
-                        else                   { b = ld16<false>(p1 + voff); if (kind != SAR_OP_COPY) a = ld16<false>(p0 + voff); }
+                        const uint32_t slots = FWD ? ops[j].slots : 0u;
+                        const bool get0 = FWD && (flags & DEVOP_GET0), get1 = FWD && (flags & DEVOP_GET1);
+                        if (get1) b = mine[(slots >> 8 & 0xffu) * BLOCK];
+                        if (get0 && kind != SAR_OP_COPY) a = mine[(slots & 0xffu) * BLOCK];
+                        if (flags & DEVOP_LNT) { if (!get1) b = ld16<true>(p1 + voff); if (!get0 && kind != SAR_OP_COPY) a = ld16<true>(p0 + voff); }
+                        else                   { if (!get1) b = ld16<false>(p1 + voff); if (!get0 && kind != SAR_OP_COPY) a = ld16<false>(p0 + voff); }
                         const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
                         if (flags & DEVOP_SNT0) st16<true>(p0 + voff, s); else st16<false>(p0 + voff, s);
                         if (kind == SAR_OP_XREDUCE) { if (flags & DEVOP_SNT1) st16<true>(p1 + voff, s); else st16<false>(p1 + voff, s); }
+                        if (FWD && (flags & DEVOP_PUT)) mine[(slots >> 16 & 0xffu) * BLOCK] = s;
                     }
                     // the < 16 bytes behind the last whole vector of the row, in the column that holds them
+                    // (always through memory: every forwarded value has been stored as well)
                     const uint64_t tail_at = bytes & ~(uint64_t)15u;
                     const uint32_t tail = (uint32_t)(bytes & 15u) / sizeof(T);
                     if (tail && tail_at >= off && tail_at < off + col_bytes && threadIdx.x < tail) {
@@ -392,31 +402,44 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
             // This round's stores are complete before this workgroup's loads of the next round.  (Lanes mostly
             // re-read what they wrote themselves, but elements change lanes between aligned and unaligned
             // rows and at partial vectors; measured, the barrier also pays for itself by keeping the waves
-            // of a workgroup on the same rows.)
-            __syncthreads();
+            // of a workgroup on the same rows.)  When the host has found that every lane only re-reads bytes
+            // it wrote itself (lane_local), program order already covers that and the waves only meet,
+            // without waiting for their stores to drain.
+            if (lane_local) __builtin_amdgcn_s_barrier(); else __syncthreads();
         }
     }
 }
 
 uint64_t column_bytes(int block) { return (uint64_t)block * 16u; }
+uint64_t column_lds_budget() { return 65536u; }
 
-template <int DT>
-static hipError_t launch_column_dt(int block, uint32_t grid, hipStream_t st, const DevOp* ops, const uint32_t* round_begin, uint32_t nrounds, uint32_t ncols) {
+template <int DT, bool FWD>
+static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, hipStream_t st, const DevOp* ops, const uint32_t* round_begin, uint32_t nrounds, uint32_t ncols, uint32_t lane_local) {
     switch (block) {
-        case 256: hipLaunchKernelGGL((column_kernel<DT, 256>), dim3(grid), dim3(256), 0, st, ops, round_begin, nrounds, ncols); break;
-        case 512: hipLaunchKernelGGL((column_kernel<DT, 512>), dim3(grid), dim3(512), 0, st, ops, round_begin, nrounds, ncols); break;
-        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024>), dim3(grid), dim3(1024), 0, st, ops, round_begin, nrounds, ncols); break;
+        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD>), dim3(grid), dim3(256), lds, st, ops, round_begin, nrounds, ncols, lane_local); break;
+        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD>), dim3(grid), dim3(512), lds, st, ops, round_begin, nrounds, ncols, lane_local); break;
+        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD>), dim3(grid), dim3(1024), lds, st, ops, round_begin, nrounds, ncols, lane_local); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-hipError_t launch_column(int dtype, int block, uint32_t grid, hipStream_t st, const DevOp* ops, const uint32_t* round_begin, uint32_t nrounds, uint32_t ncols) {
+hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, uint32_t lane_local, hipStream_t st, const DevOp* ops, const uint32_t* round_begin, uint32_t nrounds, uint32_t ncols) {
     if (ncols == 0 || grid == 0 || nrounds == 0) return hipSuccess;
+    const uint64_t lds = (uint64_t)nslots * column_bytes(block);
+    if (nslots > 255u || lds > column_lds_budget()) return hipErrorInvalidValue;
+    if (nslots) {
+        switch (dtype) {
+            case SAR_F32: return launch_column_dt<SAR_F32, true>(block, grid, (uint32_t)lds, st, ops, round_begin, nrounds, ncols, lane_local);
+            case SAR_F16: return launch_column_dt<SAR_F16, true>(block, grid, (uint32_t)lds, st, ops, round_begin, nrounds, ncols, lane_local);
+            case SAR_BF16: return launch_column_dt<SAR_BF16, true>(block, grid, (uint32_t)lds, st, ops, round_begin, nrounds, ncols, lane_local);
+            default: return hipErrorInvalidValue;
+        }
+    }
     switch (dtype) {
-        case SAR_F32: return launch_column_dt<SAR_F32>(block, grid, st, ops, round_begin, nrounds, ncols);
-        case SAR_F16: return launch_column_dt<SAR_F16>(block, grid, st, ops, round_begin, nrounds, ncols);
-        case SAR_BF16: return launch_column_dt<SAR_BF16>(block, grid, st, ops, round_begin, nrounds, ncols);
+        case SAR_F32: return launch_column_dt<SAR_F32, false>(block, grid, 0, st, ops, round_begin, nrounds, ncols, lane_local);
+        case SAR_F16: return launch_column_dt<SAR_F16, false>(block, grid, 0, st, ops, round_begin, nrounds, ncols, lane_local);
+        case SAR_BF16: return launch_column_dt<SAR_BF16, false>(block, grid, 0, st, ops, round_begin, nrounds, ncols, lane_local);
         default: return hipErrorInvalidValue;
     }
 }

@@ -11,7 +11,10 @@ enum : uint32_t {
     DEVOP_LNT = 1u,    // loads are streaming (nontemporal)
     DEVOP_SNT0 = 2u,   // stores to p0 (or to every MREDUCE destination) are streaming
     DEVOP_SNT1 = 4u,   // stores to p1 are streaming (XREDUCE only)
-    DEVOP_VEC = 8u     // every pointer of the row is 16-byte aligned
+    DEVOP_VEC = 8u,    // every pointer of the row is 16-byte aligned
+    DEVOP_GET0 = 16u,  // column executor: p0's current value is in value slot (slots & 0xff)
+    DEVOP_GET1 = 32u,  // column executor: p1's current value is in value slot (slots >> 8 & 0xff)
+    DEVOP_PUT = 64u    // column executor: keep the row's result in value slot (slots >> 16 & 0xff)
 };
 
 // One lowered row of a round, read by the kernel through scalar loads.
@@ -26,7 +29,7 @@ struct DevOp {
     uint32_t nsrc;        // MREDUCE: sources, in add order
     uint32_t ndst;        // MREDUCE: destinations
     uint32_t ptr_off;     // MREDUCE: index of srcs[0] in the pointer list; dsts follow the srcs
-    uint32_t reserved0;
+    uint32_t slots;       // column executor: value slots of DEVOP_GET0 / GET1 / PUT, one byte each
     uint64_t reserved1;
 };
 static_assert(sizeof(DevOp) == 64, "DevOp is read as one 64-byte scalar load");
@@ -40,8 +43,12 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
                           uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
 // column executor: all rounds of COPY / REDUCE_INTO / XREDUCE rows (each exactly one chunk long) in one
 // launch; rows of round r are ops[round_begin[r] .. round_begin[r+1]); a column is column_bytes(block) wide
+// With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots * column_bytes(block) bytes,
+// at most column_lds_budget()) and rows flagged DEVOP_GET* take their operands from there instead of memory.
 uint64_t column_bytes(int block);
-hipError_t launch_column(int dtype, int block, uint32_t grid, hipStream_t st, const DevOp* ops, const uint32_t* round_begin,
+uint64_t column_lds_budget();
+// lane_local != 0 promises that no lane reads bytes another lane wrote (all rows 16-byte aligned, no partial vectors).
+hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, uint32_t lane_local, hipStream_t st, const DevOp* ops, const uint32_t* round_begin,
                          uint32_t nrounds, uint32_t ncols);
 
 hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype);

@@ -192,6 +192,46 @@ def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
                     assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
 
 
+@pytest.mark.parametrize("alg,n,table", [("stragglar", 8, "stragglar_n8_cu.txt"), ("stragglar", 8, "synth_pow2_n8.txt"),
+                                         ("ring", 8, None), ("rhd", 8, None), ("direct", 8, None),
+                                         ("stragglar", 16, "synth_pow2_n16.txt"), ("stragglar", 6, "synth_nonpow2_n6.txt"),
+                                         ("ring", 16, None)])
+def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, table):
+    """The column executor may keep values a lane wrote in LDS slots and take later operands from
+    there instead of loading them again; however many slots it gets, whatever the column width and
+    barrier kind, the buffers must equal the checker's (which re-reads everything from memory)."""
+    text = read_golden(table) if table else None
+    parts = (n - 1) if alg == "stragglar" else (1 if alg == "direct" else n)
+    # whole vectors per chunk; a chunk of 4k+2 elements (partial last vector); an odd chunk (rows lose 16-byte alignment)
+    for dtype, chunk_elems in (("f32", 4096 + 512), ("f32", 4 * 700 + 2), ("bf16", 8 * 300 + 3), ("f16", 8 * 1030)):
+        elems = parts * chunk_elems + (2 if parts > 1 else 0)
+        inputs = make_inputs(n, elems, dtype, seed=21, kind="normal", scale=1.0)
+        want = run_oracle(oracle, alg, inputs, dtype, text, delay=-1.0)
+        seen = set()
+        for t in (dict(col_forward=0), dict(col_forward=1), dict(col_forward=1, col_slots=1), dict(col_forward=1, col_slots=2),
+                  dict(col_forward=1, col_slots=3, col_block=512), dict(col_forward=1, col_slots=5, col_light_sync=0),
+                  dict(col_forward=1, col_slots=16, col_block=256), dict(col_forward=1, col_slots=255, col_block=1024),
+                  dict(col_forward=1, cache_policy=0), dict(col_forward=1, cache_policy=1, col_light_sync=0)):
+            got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(t, executor=1))
+            st = gpu_ctx.stats()
+            assert st.executor == 1
+            if not t["col_forward"]:
+                assert st.forwarded_bytes == 0 and st.col_slots == 0
+            else:
+                assert st.col_slots <= min(t.get("col_slots") or 255, 65536 // (16 * st.col_block))
+                assert st.forwarded_bytes <= st.algorithmic_bytes
+                assert (st.forwarded_bytes > 0) == (st.col_slots > 0)
+            seen.add(st.forwarded_bytes)
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "%s n=%d %s chunk %d tuning %r rank %d" % (alg, n, dtype, chunk_elems, t, r))
+        es = 4 if dtype == "f32" else 2
+        if (chunk_elems * es) % 16 == 0:
+            assert max(seen) > 0, "aligned rows: some operand must have been forwarded"
+        if alg == "stragglar" and (chunk_elems * es) % 16 == 0:
+            # every re-read found in a slot: the n-1 ranks' (n-2) copies each of one chunk
+            assert max(seen) == (n - 1) * (n - 2) * chunk_elems * es
+
+
 def test_graph_replays_match_eager(gpu_ctx, sarlib, oracle):
     """The captured graph holds kernel nodes only; every replay, with eager work and synchronisation
     between replays, must equal the eager result."""
