@@ -16,6 +16,14 @@ roofline  = algorithmic bytes per launch / mean launch duration of the dominant
             with an event pair around every launch
 cpu_baseline = the CPU checker (oracle/, a port) executing the same schedule
             on the host cores of this box, on a bounded sample
+
+The column executor forwards values: a COPY whose source the same lane wrote in
+an earlier round takes it from an LDS slot instead of loading it again (every
+store still happens).  Those re-reads are part of the algorithmic bytes (each
+row is priced on its own), so `value` can pass what HBM alone could deliver;
+`forwarded_bytes_per_step`, `memory_side_GBps` and `roofline.traffic` say how
+much really went to memory, and `every_operand_loaded` repeats the measurement
+with forwarding switched off (traffic = algorithmic bytes).
 """
 import argparse
 import json
@@ -89,6 +97,8 @@ def main():
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
     ap.add_argument("--executor", type=int, default=None, choices=[0, 1, 2],
                     help="0 = one launch per round, 1 = column executor (one launch per schedule), 2 = chosen by the library's cost model (default)")
+    ap.add_argument("--forward", type=int, default=None, choices=[0, 1],
+                    help="column executor: 1 = operands a lane wrote itself come from LDS slots instead of memory (default), 0 = every operand is loaded")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build emulates all ranks on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -111,6 +121,8 @@ def main():
         main_sched, table_name = lib.builtin(args.alg, n), args.alg
     if args.executor is not None:
         ctx.set_tuning(executor=args.executor)
+    if args.forward is not None:
+        ctx.set_tuning(col_forward=args.forward)
     ctx.prepare(main_sched, None, use_graph=args.graph)
     st = ctx.stats()
     tune = ctx.get_tuning().as_dict()
@@ -153,12 +165,12 @@ def main():
     if os.path.exists(tpath):
         with open(tpath) as f:
             t = json.load(f)
-        key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, "column" if st.executor == 1 else "rounds")
+        key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, ("column_forwarding" if st.col_slots else "column") if st.executor == 1 else "rounds")
         if key in t:
             traffic = t[key]["hbm_bytes_per_launch"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                "kernel": "sar::column_kernel<f32, %d>" % st.col_block if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
+                "kernel": "sar::column_kernel<f32, %d, %s>" % (st.col_block, "forwarding" if st.col_slots else "no forwarding") if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
                 "launches": len(launch_bytes),
                 "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
     # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
@@ -171,11 +183,31 @@ def main():
                    "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph), "tuning": tune, "executor_used": "column" if st.executor == 1 else "rounds"},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
+        # part of the algorithmic bytes that never leaves the compute unit: re-reads of values the same lane wrote
+        # in an earlier round, taken from LDS slots (every store still goes to the rank buffers)
+        "forwarded_bytes_per_step": int(st.forwarded_bytes),
+        "memory_side_GBps": round((st.algorithmic_bytes - st.forwarded_bytes) / ms / 1e6, 1),
         "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),
         "wall_ms_per_step_back_to_back": round(back_to_back_ms, 4),
         "ranks_identical_after_run": bool(identical),
         "roofline": roofline,
     }
+    if st.col_slots and args.forward is None:
+        # the same steps with every operand loaded from the rank buffers (traffic = algorithmic bytes)
+        ctx.set_tuning(col_forward=0)
+        ctx.prepare(main_sched, None, use_graph=args.graph)
+        plain_ms = []
+        for i in range(args.warmup + args.steps):
+            ctx.restore()
+            t = ctx.run(-1.0)
+            if i >= args.warmup:
+                plain_ms.append(t)
+        pm = statistics.fmean(plain_ms)
+        rec["every_operand_loaded"] = {"value": round(st.algorithmic_bytes / pm / 1e6, 1), "unit": "GB/s", "ms_per_step": round(pm, 5),
+                                       "frac_of_hbm_peak": round(st.algorithmic_bytes / pm / 1e6 / HBM_PEAK_GBPS, 4),
+                                       "ranks_identical_after_run": bool(ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts))}
+        ctx.set_tuning(col_forward=1)
+        ctx.prepare(main_sched, None, use_graph=False)
     if not args.no_cpu and args.alg == "stragglar":
         from oracle import parse_table
         gold = os.path.join(ROOT, "tests", "golden", "stragglar_n%d_cu.txt" % n)

@@ -88,8 +88,11 @@ typedef struct sar_tuning_t {
     int32_t block;        /* threads per workgroup: 256 or 512                                       */
     int32_t unroll;       /* 16-byte vectors per thread and stream: 1, 2, 4 or 8                     */
     int32_t order;        /* 0 = tiles op by op, 1 = tiles of a round's ops interleaved              */
-    int32_t cache_policy; /* 0 = all accesses cached, 1 = all streaming (nontemporal), 2 = planned:  */
-                          /*     streaming unless the data is read again within `reuse_rounds`       */
+    int32_t cache_policy; /* 0 = all accesses cached, 1 = all streaming (nontemporal), 3 = streaming */
+                          /*     loads and cached stores, 2 = planned (default).  One launch per     */
+                          /*     round plans per row: streaming unless the data is read again within */
+                          /*     `reuse_rounds`.  The column executor has one policy per launch: it  */
+                          /*     plans streaming loads when values are forwarded, else all cached    */
     int32_t reuse_rounds; /* look-ahead of policy 2, in rounds                                       */
     int32_t reverse_odd;  /* 1 = odd rounds walk their tiles backwards (keeps the cache tail warm)   */
     int32_t segments;     /* >1: cut every row into this many pieces and run the whole schedule      */
@@ -109,6 +112,9 @@ typedef struct sar_tuning_t {
     int32_t col_light_sync; /* column executor: 1 = between rounds the waves of a workgroup only meet   */
                           /*     (no wait for their stores) whenever no lane reads bytes another lane */
                           /*     wrote; 0 = always a full barrier                                     */
+    int32_t col_latency_plan; /* column executor: the plan for few columns (row table copied into LDS, the  */
+                          /*     inputs of the first rows fetched into slots before round 0): 0 = never,  */
+                          /*     1 = when there are at most two columns per compute unit, 2 = always      */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

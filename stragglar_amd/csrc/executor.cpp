@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -69,7 +69,7 @@ struct sar_ctx {
     // column plan (tune.executor == 1): the whole main schedule as one launch
     bool column = false;
     uint32_t* d_round_begin = nullptr;
-    uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512, col_slots = 0, col_lane_local = 0;
+    uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512, col_slots = 0, col_lane_local = 0, col_staged_rows = 0, col_policy = 0;
     int cu_count = 0;
 
     std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
@@ -88,7 +88,7 @@ void drop_plan(sar_ctx* c) {
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
     if (c->d_round_begin) { (void)hipFree(c->d_round_begin); c->d_round_begin = nullptr; }
-    c->column = false; c->col_rounds = c->col_count = c->col_grid = c->col_slots = 0;
+    c->column = false; c->col_rounds = c->col_count = c->col_grid = c->col_slots = c->col_staged_rows = c->col_policy = 0;
     c->prework.clear(); c->rounds.clear(); c->prepared = false;
     c->stats = sar_stats_t{};
 }
@@ -240,6 +240,8 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
             const RowAccess& ra = acc[ri][oi];
             if (c->tune.cache_policy == 1) {
                 d.flags |= sar::DEVOP_LNT | sar::DEVOP_SNT0 | sar::DEVOP_SNT1;
+            } else if (c->tune.cache_policy == 3) {
+                d.flags |= sar::DEVOP_LNT;
             } else if (c->tune.cache_policy == 2) {
                 bool any_read_again = false;
                 for (const auto& rd : ra.reads) any_read_again |= read_soon(ri, rd);
@@ -289,8 +291,7 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
 // for one value and the set of cells that currently equal it (a COPY from a held value adds its
 // destination to the set at no cost; a write to a cell takes it out of its old set).  When all slots
 // are busy the value whose next use is furthest away gives way, which is known exactly because the
-// whole schedule is.  Rows get DEVOP_GET0 / GET1 / PUT and their slot numbers; the cache policy is
-// then planned on the reads that still go to memory.
+// whole schedule is.  Rows get DEVOP_GET0 / GET1 / PUT and their slot numbers.
 struct ColumnPlan {
     std::vector<uint32_t> round_begin;
     uint64_t widest_row = 0;
@@ -298,6 +299,8 @@ struct ColumnPlan {
     uint32_t nslots = 0;
     uint64_t forwarded_bytes = 0;    // operand bytes taken from value slots instead of memory, per run
     bool lane_local = false;         // every row 16-byte aligned and a whole number of vectors long
+    bool staged = false;             // latency plan: the workgroups copy the row table into LDS first
+    uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
 };
 
 int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, ColumnPlan& plan) {
@@ -342,6 +345,22 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
 
     // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
     plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512) >= 2048 ? 512 : 256);
+
+    // Latency plan: when the columns are so few that they are all resident at once, time goes into dependent round
+    // trips, not bandwidth, and nobody warms the scalar cache: a row read through scalar loads is a trip to L2.  The
+    // workgroups then copy the row table into LDS first.  Forwarding is left out of it: measured, a row whose
+    // operand comes from a slot is no faster there than one whose operand comes from L2.
+    {
+        const int lb = sar::column_latency_block();
+        const uint64_t lcols = (plan.widest_row + sar::column_bytes(lb) - 1) / sar::column_bytes(lb);
+        const bool few = c->tune.col_latency_plan == 2 || (c->tune.col_latency_plan == 1 && lcols <= 2u * (uint64_t)std::max(1, c->cu_count));
+        if (few && (c->tune.col_block == 0 || c->tune.col_block == lb) &&
+            sar::column_table_bytes(nrows, (uint32_t)plan.round_begin.size() - 1) <= sar::column_lds_budget()) {
+            plan.staged = true;
+            plan.block = lb;
+        }
+    }
+
     // per cell, the rows that touch it, in order; a reducing row reads and writes its cell
     const int ncells = c->n * cells_per_rank;
     struct Ev { uint32_t row; bool reads, writes; };
@@ -432,55 +451,37 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
         return f;
     };
 
-    // How many slots.  LDS per compute unit is what they cost: up to 5 per lane all 2048 lanes of a compute unit
-    // stay resident, up to 10 half of them.  Measured on MI355X, half occupancy pays when every re-read is then
-    // found in a slot (what still goes to memory is the cold inputs and the stores), but not for a part of them;
-    // and a plan that finds less than a tenth of the bytes the rows move is not worth the longer row loop.
-    Forwarding fwd;
-    if (c->tune.col_forward) {
+    Forwarding fwd = forward(0);
+    bool all_found = false;              // every re-read of the column finds its operand in a slot
+    if (c->tune.col_forward && !plan.staged) {
         const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, sar::column_lds_budget() / sar::column_bytes(plan.block));
         if (c->tune.col_slots > 0) {
             fwd = forward(std::min<uint32_t>(fit, (uint32_t)c->tune.col_slots));
+            all_found = fwd.nslots && fwd.bytes == forward(255u).bytes;
         } else {
+            // How many slots.  LDS per compute unit is what they cost: up to 5 per lane all 2048 lanes of a compute
+            // unit stay resident, up to 10 half of them.  Measured on MI355X, half occupancy pays when every re-read
+            // is then found in a slot (what still goes to memory is the cold inputs and the stores), but not for a
+            // part of them; and a plan that finds less than a tenth of the bytes the rows move is not worth the
+            // longer row loop.
             const uint64_t all = forward(255u).bytes;
             fwd = forward(std::min<uint32_t>(fit, 10u));
             if (fwd.bytes != all) fwd = forward(std::min<uint32_t>(fit, 5u));
+            all_found = fwd.nslots && fwd.bytes == all;
             uint64_t moved = 0;                  // algorithmic bytes of the rows
             for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : 3u);
             if (fwd.bytes * 10u < moved) fwd = forward(0);
         }
-    } else {
-        fwd = forward(0);
     }
     plan.nslots = fwd.nslots; plan.forwarded_bytes = fwd.bytes;
-    std::vector<uint8_t> memread0(nrows, 0), memread1(nrows, 0);
-    for (uint32_t i = 0; i < nrows; ++i) {
-        cr[i].d.flags |= fwd.flags[i]; cr[i].d.slots = fwd.slots[i];
-        memread0[i] = cr[i].d.kind != SAR_OP_COPY && !(fwd.flags[i] & sar::DEVOP_GET0);
-        memread1[i] = !(fwd.flags[i] & sar::DEVOP_GET1);
-    }
+    for (uint32_t i = 0; i < nrows; ++i) { cr[i].d.flags |= fwd.flags[i]; cr[i].d.slots = fwd.slots[i]; }
 
-    // Cache policy over the accesses that go to memory.  Without forwarding a column keeps its data close for the
-    // whole schedule: anything read again in ANY later row stays cached.  With forwarding what is left is mostly
-    // read or written once, and streaming everything measured faster also for the re-reads that found no slot.
-    if (c->tune.cache_policy == 1 || (c->tune.cache_policy == 2 && plan.nslots > 0)) {
-        for (auto& r : cr) r.d.flags |= sar::DEVOP_LNT | sar::DEVOP_SNT0 | sar::DEVOP_SNT1;
-    } else if (c->tune.cache_policy == 2) {
-        std::vector<uint8_t> read_later((size_t)ncells, 0);
-        // rows of one round neither read what another row of the round writes, so "later" may go row by row
-        for (uint32_t i = nrows; i-- > 0;) {
-            sar::DevOp& d = cr[i].d;
-            const int c0 = cr[i].c0, c1 = cr[i].c1;
-            bool again = false;
-            if (memread0[i]) again |= read_later[(size_t)c0] != 0;
-            if (memread1[i]) again |= read_later[(size_t)c1] != 0;
-            if (!again) d.flags |= sar::DEVOP_LNT;
-            if (!read_later[(size_t)c0]) d.flags |= sar::DEVOP_SNT0;
-            if (d.kind == SAR_OP_XREDUCE && !read_later[(size_t)c1]) d.flags |= sar::DEVOP_SNT1;
-            if (memread0[i]) read_later[(size_t)c0] = 1;
-            if (memread1[i]) read_later[(size_t)c1] = 1;
-        }
-    }
+    // Cache policy of the launch (the column kernel takes one for all its rows).  Planned (2): when every re-read is
+    // forwarded, what is still loaded is read exactly once: streaming loads (+1.5 % for the StragglAR table);
+    // otherwise the re-reads are meant to find their data in the caches and nothing streams (streaming loads cost
+    // 4-10 % there).  Streaming stores never paid in this kernel (-3 to -25 %).
+    plan.policy = c->tune.cache_policy == 0 ? 0u : c->tune.cache_policy == 1 ? 2u : c->tune.cache_policy == 3 ? 1u : (all_found ? 1u : 0u);
+
     plan.lane_local = true;
     for (const auto& r : cr) {
         if (!(r.d.flags & sar::DEVOP_VEC) || (r.d.bytes & 15u)) plan.lane_local = false;
@@ -496,9 +497,18 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
 // bytes that still go to memory: 5.0 TB/s when they are mostly stores (three tenths or more of the
 // operands found in slots), 6.0 otherwise.  A workgroup needs about 0.6 us per row while everything
 // stays cache resident, 0.95 us beyond that; one launch per round moves 6.5 TB/s and costs about 3 us
-// per launch.
+// per launch.  With the row table in LDS (latency plan) a row costs 0.32-0.65 us.
 bool column_pays(const sar_ctx* c, size_t column_rows, const ColumnPlan& cp) {
     const double bytes = (double)c->stats.algorithmic_bytes;
+    double est_rounds = 0;
+    for (const auto& L : c->rounds) if (L.total_tiles) est_rounds += 3.0 + (double)L.algorithmic_bytes / 6.5e6;
+    if (cp.staged) {
+        // latency plan: a row costs a round trip to where its data is (0.32 us while the buffers are tiny, 0.45 us
+        // while they fit the L2s, 0.65 us beyond)
+        const double resident_bytes = (double)c->bytes_per_rank * c->n;
+        const double per_row_us = resident_bytes <= 262144.0 ? 0.32 : resident_bytes <= 33554432.0 ? 0.45 : 0.65;
+        return 4.0 + std::max((double)column_rows * per_row_us, bytes / 5.5e6) <= est_rounds;
+    }
     const uint64_t cb = sar::column_bytes(cp.block);
     const double ncols = (double)((cp.widest_row + cb - 1) / cb);
     double wgs_per_cu = 2048.0 / cp.block;
@@ -514,13 +524,15 @@ bool column_pays(const sar_ctx* c, size_t column_rows, const ColumnPlan& cp) {
         est_stream = bytes / (column_rows <= 128 ? 7.1e6 : column_rows <= 256 ? 6.4e6 : 5.3e6);
     }
     const double est_column = std::max(est_stream, (double)column_rows * per_row_us * passes) + 4.0;
-    double est_rounds = 0;
-    for (const auto& L : c->rounds) if (L.total_tiles) est_rounds += 3.0 + (double)L.algorithmic_bytes / 6.5e6;
     return est_column <= est_rounds;
 }
 
 int launch_column_once(sar_ctx* c) {
-    SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->col_slots, c->col_lane_local, c->stream, c->d_ops + c->col_first_op, c->d_round_begin, c->col_rounds, c->col_count));
+    sar::ColumnLaunch L{};
+    L.ops = c->d_ops + c->col_first_op; L.round_begin = c->d_round_begin;
+    L.nrounds = c->col_rounds; L.ncols = c->col_count;
+    L.staged_rows = c->col_staged_rows; L.lane_local = c->col_lane_local; L.policy = c->col_policy;
+    SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->col_slots, c->stream, L));
     return SAR_OK;
 }
 
@@ -544,12 +556,12 @@ int launch_main(sar_ctx* c) { return c->column ? launch_column_once(c) : launch_
 
 bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
-           (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 2 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
+           (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 3 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
            (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256 &&
            (t.executor >= 0 && t.executor <= 2) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
            (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024) &&
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
-           (t.col_light_sync == 0 || t.col_light_sync == 1);
+           (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2;
 }
 
 }  // namespace
@@ -883,6 +895,8 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
         c->col_block = (uint32_t)cp.block;
         c->col_slots = cp.nslots;
         c->col_lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
+        c->col_staged_rows = cp.staged ? (uint32_t)(rows.size() - col_first) : 0u;
+        c->col_policy = cp.policy;
         const uint64_t cb = sar::column_bytes(cp.block);
         const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
         if (ncols > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 columns"); }

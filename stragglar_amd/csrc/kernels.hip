@@ -9,6 +9,7 @@
 // independent vectors in flight per lane and stream, one tile per workgroup so
 // that the hardware dispatcher balances rows of different cost.
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "kernels.hpp"
@@ -20,15 +21,19 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 
 // ---- cache-policy aware 16-byte accesses --------------------------------
+// Rank buffers are device memory: saying so (address space 1) keeps these global_load / global_store
+// instructions also where the pointer was rebuilt from integers (a flat access would tie up the LDS
+// counter as well and serialise against the LDS traffic of the column kernel).
+typedef __attribute__((address_space(1))) f4 gf4;
 template <bool NT>
 __device__ __forceinline__ f4 ld16(const char* p) {
-    const f4* q = reinterpret_cast<const f4*>(p);
+    const gf4* q = (const gf4*)p;
     if (NT) return __builtin_nontemporal_load(q);
     return *q;
 }
 template <bool NT>
 __device__ __forceinline__ void st16(char* p, f4 v) {
-    f4* q = reinterpret_cast<f4*>(p);
+    gf4* q = (gf4*)p;
     if (NT) __builtin_nontemporal_store(v, q);
     else *q = v;
 }
@@ -349,37 +354,86 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // One row at a time and one vector per lane turned out best (28 VGPRs, eight waves per SIMD resident:
 // the other workgroups of the compute unit cover a row's latency; batching the loads of several rows or
 // several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
-template <int DT, int BLOCK, bool FWD>
-__global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ round_begin,
-                                                        uint32_t nrounds, uint32_t ncols, uint32_t lane_local) {
+// One row as the column kernel uses it, every field wave-uniform (SGPRs).
+struct ColRow { char* p0; char* p1; uint64_t bytes; uint32_t kind, flags, slots; };
+
+__device__ __forceinline__ uint32_t uniform32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+// Row j of the launch: from the copy of the row table in LDS when there is one (a broadcast read, made
+// uniform again with readfirstlane), else through scalar loads from memory.
+template <bool STAGED>
+__device__ __forceinline__ ColRow column_row(const DevOp* __restrict__ ops, const u4* table, uint32_t j) {
+    ColRow r;
+    if (STAGED) {
+        const u4 q0 = table[j * 4u], q1 = table[j * 4u + 1u], q3 = table[j * 4u + 3u];
+        r.p0 = reinterpret_cast<char*>((uint64_t)uniform32(q0.x) | ((uint64_t)uniform32(q0.y) << 32));
+        r.p1 = reinterpret_cast<char*>((uint64_t)uniform32(q0.z) | ((uint64_t)uniform32(q0.w) << 32));
+        r.bytes = (uint64_t)uniform32(q1.x) | ((uint64_t)uniform32(q1.y) << 32);
+        r.kind = uniform32(q1.z); r.flags = uniform32(q1.w); r.slots = uniform32(q3.y);
+    } else {
+        r.p0 = ops[j].p0; r.p1 = ops[j].p1; r.bytes = ops[j].bytes;
+        r.kind = ops[j].kind; r.flags = ops[j].flags; r.slots = ops[j].slots;
+    }
+    return r;
+}
+static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offsetof(DevOp, kind) == 24 &&
+              offsetof(DevOp, flags) == 28 && offsetof(DevOp, slots) == 52, "column_row reads DevOp by position");
+
+// FWD: value slots in LDS (rows flagged DEVOP_GET* / DEVOP_PUT).  LAT: the plan for few columns -- the row
+// table is copied into LDS first (never together with FWD).  POL: cache policy of the whole launch, 0 = all
+// accesses cached, 1 = streaming (nontemporal) loads and cached stores, 2 = streaming loads and stores.  The
+// policy is a template argument because a flavour picked per row at run time does not survive compilation:
+// the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.
+template <int DT, int BLOCK, bool FWD, bool LAT, int POL>
+__global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ round_begin, ColumnLaunch L) {
     typedef typename Elem<DT>::T T;
+    static_assert(!(FWD && LAT), "the latency plan does not forward");
     constexpr uint64_t col_bytes = (uint64_t)BLOCK * 16u;
-    // FWD: value slots in LDS, slot k of lane t at vector k*BLOCK + t.  A lane only ever touches its
-    // own vectors, so the slots need no synchronisation of their own.
+    constexpr bool LNT = POL >= 1, SNT = POL == 2;
+    // LDS: LAT: [copy of the row table: staged_rows x 64 B][copy of round_begin]; FWD: the value slots, slot k of
+    // lane t at vector k*BLOCK + t.  A lane only ever touches its own vectors, so the slots need no
+    // synchronisation of their own.
+    // (the two tables come as kernel arguments of their own: only a __restrict__ const parameter lets the
+    // compiler read them through scalar loads)
     extern __shared__ __align__(16) char lds_raw[];
+    const u4* table = nullptr;
+    const uint32_t* rbegin = round_begin;
+    if (LAT) {
+        // Few workgroups, nobody to warm the scalar cache: a row read through scalar loads costs a trip to L2
+        // (about half a microsecond) and the rows come one after the other.  Fetch the whole table at once.
+        const uint32_t table_vecs = L.staged_rows * 4u;
+        u4* dst = reinterpret_cast<u4*>(lds_raw);
+        const u4* src = reinterpret_cast<const u4*>(ops);
+        for (uint32_t i = threadIdx.x; i < table_vecs; i += BLOCK) dst[i] = src[i];
+        uint32_t* bdst = reinterpret_cast<uint32_t*>(lds_raw) + table_vecs * 4u;
+        for (uint32_t i = threadIdx.x; i <= L.nrounds; i += BLOCK) bdst[i] = round_begin[i];
+        __syncthreads();
+        table = reinterpret_cast<const u4*>(lds_raw);
+        rbegin = bdst;
+    }
     f4* const mine = reinterpret_cast<f4*>(lds_raw) + threadIdx.x;
-    for (uint32_t col = blockIdx.x; col < ncols; col += gridDim.x) {
+    for (uint32_t col = blockIdx.x; col < L.ncols; col += gridDim.x) {
         const uint64_t off = (uint64_t)col * col_bytes;
         const uint64_t voff = off + ((uint64_t)threadIdx.x << 4);       // this lane's vector within every row
-        for (uint32_t r = 0; r < nrounds; ++r) {
-            const uint32_t rb = round_begin[r], re = round_begin[r + 1];
+        for (uint32_t r = 0; r < L.nrounds; ++r) {
+            uint32_t rb, re;
+            if (LAT) { rb = uniform32(rbegin[r]); re = uniform32(rbegin[r + 1u]); } else { rb = rbegin[r]; re = rbegin[r + 1u]; }
             for (uint32_t j = rb; j < re; ++j) {
-                const uint32_t flags = ops[j].flags, kind = ops[j].kind;
-                const uint64_t bytes = ops[j].bytes;
-                char* const p0 = ops[j].p0;
-                char* const p1 = ops[j].p1;
+                const ColRow row = column_row<LAT>(ops, table, j);
+                const uint32_t flags = row.flags, kind = row.kind;
+                const uint64_t bytes = row.bytes;
+                char* const p0 = row.p0;
+                char* const p1 = row.p1;
                 if (flags & DEVOP_VEC) {
                     if (voff + 16u <= bytes) {
                         f4 a = {0.f, 0.f, 0.f, 0.f}, b;
-                        const uint32_t slots = FWD ? ops[j].slots : 0u;
+                        const uint32_t slots = FWD ? row.slots : 0u;
                         const bool get0 = FWD && (flags & DEVOP_GET0), get1 = FWD && (flags & DEVOP_GET1);
-                        if (get1) b = mine[(slots >> 8 & 0xffu) * BLOCK];
-                        if (get0 && kind != SAR_OP_COPY) a = mine[(slots & 0xffu) * BLOCK];
-                        if (flags & DEVOP_LNT) { if (!get1) b = ld16<true>(p1 + voff); if (!get0 && kind != SAR_OP_COPY) a = ld16<true>(p0 + voff); }
-                        else                   { if (!get1) b = ld16<false>(p1 + voff); if (!get0 && kind != SAR_OP_COPY) a = ld16<false>(p0 + voff); }
+                        if (get1) b = mine[(slots >> 8 & 0xffu) * BLOCK]; else b = ld16<LNT>(p1 + voff);
+                        if (kind != SAR_OP_COPY) { if (get0) a = mine[(slots & 0xffu) * BLOCK]; else a = ld16<LNT>(p0 + voff); }
                         const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
-                        if (flags & DEVOP_SNT0) st16<true>(p0 + voff, s); else st16<false>(p0 + voff, s);
-                        if (kind == SAR_OP_XREDUCE) { if (flags & DEVOP_SNT1) st16<true>(p1 + voff, s); else st16<false>(p1 + voff, s); }
+                        st16<SNT>(p0 + voff, s);
+                        if (kind == SAR_OP_XREDUCE) st16<SNT>(p1 + voff, s);
                         if (FWD && (flags & DEVOP_PUT)) mine[(slots >> 16 & 0xffu) * BLOCK] = s;
                     }
                     // the < 16 bytes behind the last whole vector of the row, in the column that holds them
@@ -405,41 +459,55 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
             // of a workgroup on the same rows.)  When the host has found that every lane only re-reads bytes
             // it wrote itself (lane_local), program order already covers that and the waves only meet,
             // without waiting for their stores to drain.
-            if (lane_local) __builtin_amdgcn_s_barrier(); else __syncthreads();
+            if (L.lane_local) __builtin_amdgcn_s_barrier(); else __syncthreads();
         }
     }
 }
 
 uint64_t column_bytes(int block) { return (uint64_t)block * 16u; }
 uint64_t column_lds_budget() { return 65536u; }
+uint64_t column_table_bytes(uint32_t rows, uint32_t nrounds) { return (uint64_t)rows * sizeof(DevOp) + (((uint64_t)nrounds + 1u + 3u) / 4u) * 16u; }
+int column_latency_block() { return 256; }
 
-template <int DT, bool FWD>
-static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, hipStream_t st, const DevOp* ops, const uint32_t* round_begin, uint32_t nrounds, uint32_t ncols, uint32_t lane_local) {
+template <int DT, bool FWD, int POL>
+static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hipStream_t st, const ColumnLaunch& L) {
     switch (block) {
-        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD>), dim3(grid), dim3(256), lds, st, ops, round_begin, nrounds, ncols, lane_local); break;
-        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD>), dim3(grid), dim3(512), lds, st, ops, round_begin, nrounds, ncols, lane_local); break;
-        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD>), dim3(grid), dim3(1024), lds, st, ops, round_begin, nrounds, ncols, lane_local); break;
+        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.round_begin, L); break;
+        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL>), dim3(grid), dim3(512), lds, st, L.ops, L.round_begin, L); break;
+        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL>), dim3(grid), dim3(1024), lds, st, L.ops, L.round_begin, L); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, uint32_t lane_local, hipStream_t st, const DevOp* ops, const uint32_t* round_begin, uint32_t nrounds, uint32_t ncols) {
-    if (ncols == 0 || grid == 0 || nrounds == 0) return hipSuccess;
-    const uint64_t lds = (uint64_t)nslots * column_bytes(block);
-    if (nslots > 255u || lds > column_lds_budget()) return hipErrorInvalidValue;
-    if (nslots) {
-        switch (dtype) {
-            case SAR_F32: return launch_column_dt<SAR_F32, true>(block, grid, (uint32_t)lds, st, ops, round_begin, nrounds, ncols, lane_local);
-            case SAR_F16: return launch_column_dt<SAR_F16, true>(block, grid, (uint32_t)lds, st, ops, round_begin, nrounds, ncols, lane_local);
-            case SAR_BF16: return launch_column_dt<SAR_BF16, true>(block, grid, (uint32_t)lds, st, ops, round_begin, nrounds, ncols, lane_local);
-            default: return hipErrorInvalidValue;
-        }
+template <int DT, int POL>
+static hipError_t launch_column_policy(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
+    if (L.staged_rows) {
+        hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.round_begin, L);
+        return hipGetLastError();
     }
+    return fwd ? launch_column_block<DT, true, POL>(block, grid, lds, st, L) : launch_column_block<DT, false, POL>(block, grid, lds, st, L);
+}
+
+template <int DT>
+static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
+    switch (L.policy) {
+        case 0: return launch_column_policy<DT, 0>(block, grid, lds, fwd, st, L);
+        case 1: return launch_column_policy<DT, 1>(block, grid, lds, fwd, st, L);
+        case 2: return launch_column_policy<DT, 2>(block, grid, lds, fwd, st, L);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, hipStream_t st, const ColumnLaunch& L) {
+    if (L.ncols == 0 || grid == 0 || L.nrounds == 0) return hipSuccess;
+    const bool lat = L.staged_rows != 0;
+    const uint64_t lds = lat ? column_table_bytes(L.staged_rows, L.nrounds) : (uint64_t)nslots * column_bytes(block);
+    if (nslots > 255u || lds > column_lds_budget() || (lat && (nslots || block != column_latency_block()))) return hipErrorInvalidValue;
     switch (dtype) {
-        case SAR_F32: return launch_column_dt<SAR_F32, false>(block, grid, 0, st, ops, round_begin, nrounds, ncols, lane_local);
-        case SAR_F16: return launch_column_dt<SAR_F16, false>(block, grid, 0, st, ops, round_begin, nrounds, ncols, lane_local);
-        case SAR_BF16: return launch_column_dt<SAR_BF16, false>(block, grid, 0, st, ops, round_begin, nrounds, ncols, lane_local);
+        case SAR_F32: return launch_column_dt<SAR_F32>(block, grid, (uint32_t)lds, nslots != 0, st, L);
+        case SAR_F16: return launch_column_dt<SAR_F16>(block, grid, (uint32_t)lds, nslots != 0, st, L);
+        case SAR_BF16: return launch_column_dt<SAR_BF16>(block, grid, (uint32_t)lds, nslots != 0, st, L);
         default: return hipErrorInvalidValue;
     }
 }

@@ -42,14 +42,25 @@ uint64_t mreduce_tile_bytes();
 hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t nops, char* const* ptrs,
                           uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
 // column executor: all rounds of COPY / REDUCE_INTO / XREDUCE rows (each exactly one chunk long) in one
-// launch; rows of round r are ops[round_begin[r] .. round_begin[r+1]); a column is column_bytes(block) wide
-// With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots * column_bytes(block) bytes,
-// at most column_lds_budget()) and rows flagged DEVOP_GET* take their operands from there instead of memory.
+// launch; a column is column_bytes(block) wide.
+struct ColumnLaunch {
+    const DevOp* ops;            // the rows of all rounds
+    const uint32_t* round_begin; // rows of round r are ops[round_begin[r] .. round_begin[r+1])
+    uint32_t nrounds, ncols;
+    uint32_t staged_rows;        // 0, or the total number of rows: latency plan, the workgroup copies the table into
+                                 // LDS first (block = column_latency_block(), no value slots)
+    uint32_t lane_local;         // != 0 promises that no lane reads bytes another lane wrote (all rows 16-byte
+                                 // aligned, no partial vectors): rounds are then separated by an execution barrier only
+    uint32_t policy;             // whole launch: 0 = cached accesses, 1 = streaming loads, 2 = streaming loads and stores
+};
+// With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots * column_bytes(block) bytes) and
+// rows flagged DEVOP_GET* take their operands from there instead of memory.  Slots, or the staged table
+// (column_table_bytes), must fit column_lds_budget().
 uint64_t column_bytes(int block);
 uint64_t column_lds_budget();
-// lane_local != 0 promises that no lane reads bytes another lane wrote (all rows 16-byte aligned, no partial vectors).
-hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, uint32_t lane_local, hipStream_t st, const DevOp* ops, const uint32_t* round_begin,
-                         uint32_t nrounds, uint32_t ncols);
+uint64_t column_table_bytes(uint32_t rows, uint32_t nrounds);
+int column_latency_block();
+hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, hipStream_t st, const ColumnLaunch& L);
 
 hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype);
 hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype);

@@ -185,7 +185,7 @@ def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
                         assert_bits_equal(got[r], want[r], "tuning %r rank %d" % (t, r))
     for col_block in (256, 512, 1024):
         for col_wgs in (1, 4, 64, 4096):
-            for policy in (0, 1, 2):
+            for policy in (0, 1, 2, 3):
                 t = dict(executor=1, col_block=col_block, col_wgs=col_wgs, cache_policy=policy)
                 got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, None, delay=0.0, tuning=t)
                 for r in range(n):
@@ -211,16 +211,21 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
         for t in (dict(col_forward=0), dict(col_forward=1), dict(col_forward=1, col_slots=1), dict(col_forward=1, col_slots=2),
                   dict(col_forward=1, col_slots=3, col_block=512), dict(col_forward=1, col_slots=5, col_light_sync=0),
                   dict(col_forward=1, col_slots=16, col_block=256), dict(col_forward=1, col_slots=255, col_block=1024),
-                  dict(col_forward=1, cache_policy=0), dict(col_forward=1, cache_policy=1, col_light_sync=0)):
-            got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(t, executor=1))
+                  dict(col_forward=1, cache_policy=0), dict(col_forward=1, cache_policy=1, col_light_sync=0),
+                  dict(col_forward=1, cache_policy=3), dict(col_forward=0, cache_policy=3),
+                  dict(col_forward=1, col_latency_plan=1), dict(col_forward=1, col_latency_plan=2, col_slots=2),
+                  dict(col_forward=0, col_latency_plan=2, cache_policy=1)):
+            # these buffers have few columns: unless a case asks for it, keep the plan for few columns (which does
+            # not forward) out of the way
+            got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(dict(col_latency_plan=0), **dict(t, executor=1)))
             st = gpu_ctx.stats()
             assert st.executor == 1
-            if not t["col_forward"]:
+            if not t["col_forward"] or t.get("col_latency_plan"):
                 assert st.forwarded_bytes == 0 and st.col_slots == 0
             else:
                 assert st.col_slots <= min(t.get("col_slots") or 255, 65536 // (16 * st.col_block))
                 assert st.forwarded_bytes <= st.algorithmic_bytes
-                assert (st.forwarded_bytes > 0) == (st.col_slots > 0)
+                assert st.forwarded_bytes == 0 or st.col_slots > 0
             seen.add(st.forwarded_bytes)
             for r in range(n):
                 assert_bits_equal(got[r], want[r], "%s n=%d %s chunk %d tuning %r rank %d" % (alg, n, dtype, chunk_elems, t, r))
@@ -230,6 +235,23 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
         if alg == "stragglar" and (chunk_elems * es) % 16 == 0:
             # every re-read found in a slot: the n-1 ranks' (n-2) copies each of one chunk
             assert max(seen) == (n - 1) * (n - 2) * chunk_elems * es
+
+
+@pytest.mark.parametrize("alg", ["stragglar", "ring", "rhd", "direct"])
+def test_latency_plan_on_many_columns(gpu_ctx, sarlib, oracle, alg):
+    """The plan for few columns (row table copied into LDS) forced onto a buffer with many columns and few
+    workgroups, so that every workgroup walks several columns with its copy of the table."""
+    n, dtype = 8, "f32"
+    parts = 7 if alg == "stragglar" else (1 if alg == "direct" else 8)
+    elems = parts * (40 * 1024 + 4) + 3
+    inputs = make_inputs(n, elems, dtype, seed=33)
+    want = run_oracle(oracle, alg, inputs, dtype, read_golden("stragglar_n8_cu.txt") if alg == "stragglar" else None, delay=-1.0)
+    for t in (dict(col_latency_plan=2, col_wgs=1), dict(col_latency_plan=2, col_wgs=1, col_block=512),
+              dict(col_latency_plan=2, col_forward=0, cache_policy=3), dict(col_latency_plan=0)):
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, read_golden("stragglar_n8_cu.txt") if alg == "stragglar" else None,
+                      delay=-1.0, tuning=dict(t, executor=1))
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s tuning %r rank %d" % (alg, t, r))
 
 
 def test_graph_replays_match_eager(gpu_ctx, sarlib, oracle):
