@@ -348,12 +348,15 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // Rows move whole chunks, so an element only ever meets the elements at its own offset within a
 // chunk: the schedule falls apart into independent "columns" (one range of within-chunk offsets each).
 // A workgroup owns a column of BLOCK 16-byte vectors and walks ALL rounds for it, row after row, with
-// nothing but a workgroup barrier between rounds.  Every row still performs its own loads and stores on
-// the rank buffers, in schedule order for each element; but what a later round re-reads was written by
-// the same compute unit moments ago and comes from L2 / Infinity Cache instead of HBM.
-// One row at a time and one vector per lane turned out best (28 VGPRs, eight waves per SIMD resident:
-// the other workgroups of the compute unit cover a row's latency; batching the loads of several rows or
-// several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
+// nothing but a workgroup barrier between rounds.  Every row performs its stores on the rank buffers,
+// in schedule order for each element.  What a later round re-reads was written by the same lane moments
+// ago: without forwarding it comes back from L2 / Infinity Cache instead of HBM; with forwarding (FWD)
+// the lane kept it in an LDS value slot that the host assigned when it lowered the schedule, and the
+// load is not issued at all.
+// One row at a time and one vector per lane turned out best (32-38 VGPRs, eight waves per SIMD
+// resident: the other workgroups of the compute unit cover a row's latency; batching the loads of
+// several rows or several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
+
 // One row as the column kernel uses it, every field wave-uniform (SGPRs).
 struct ColRow { char* p0; char* p1; uint64_t bytes; uint32_t kind, flags, slots; };
 
@@ -426,15 +429,22 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                 char* const p1 = row.p1;
                 if (flags & DEVOP_VEC) {
                     if (voff + 16u <= bytes) {
-                        f4 a = {0.f, 0.f, 0.f, 0.f}, b;
                         const uint32_t slots = FWD ? row.slots : 0u;
                         const bool get0 = FWD && (flags & DEVOP_GET0), get1 = FWD && (flags & DEVOP_GET1);
-                        if (get1) b = mine[(slots >> 8 & 0xffu) * BLOCK]; else b = ld16<LNT>(p1 + voff);
-                        if (kind != SAR_OP_COPY) { if (get0) a = mine[(slots & 0xffu) * BLOCK]; else a = ld16<LNT>(p0 + voff); }
-                        const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
-                        st16<SNT>(p0 + voff, s);
-                        if (kind == SAR_OP_XREDUCE) st16<SNT>(p1 + voff, s);
-                        if (FWD && (flags & DEVOP_PUT)) mine[(slots >> 16 & 0xffu) * BLOCK] = s;
+                        if (FWD && kind == SAR_OP_COPY && get1) {
+                            // A copy of a held value is a store and nothing else.  It has a path of its own so
+                            // that it does not pass the wait for loaded operands below: the memory counter
+                            // runs in order, and that wait would also sit out the stores of the rows before.
+                            st16<SNT>(p0 + voff, mine[(slots >> 8 & 0xffu) * BLOCK]);
+                        } else {
+                            f4 a = {0.f, 0.f, 0.f, 0.f}, b;
+                            if (get1) b = mine[(slots >> 8 & 0xffu) * BLOCK]; else b = ld16<LNT>(p1 + voff);
+                            if (kind != SAR_OP_COPY) { if (get0) a = mine[(slots & 0xffu) * BLOCK]; else a = ld16<LNT>(p0 + voff); }
+                            const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
+                            st16<SNT>(p0 + voff, s);
+                            if (kind == SAR_OP_XREDUCE) st16<SNT>(p1 + voff, s);
+                            if (FWD && (flags & DEVOP_PUT)) mine[(slots >> 16 & 0xffu) * BLOCK] = s;
+                        }
                     }
                     // the < 16 bytes behind the last whole vector of the row, in the column that holds them
                     // (always through memory: every forwarded value has been stored as well)
