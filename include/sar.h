@@ -83,7 +83,7 @@ typedef struct sar_stats_t {
                                    /* in LDS instead of loading it again from the rank buffers                    */
 } sar_stats_t;
 
-/* run-time tunables of the round kernel; sar_get_tuning() reports the defaults */
+/* run-time tunables of the executors; sar_get_tuning() reports the defaults */
 typedef struct sar_tuning_t {
     int32_t block;        /* threads per workgroup: 256 or 512                                       */
     int32_t unroll;       /* 16-byte vectors per thread and stream: 1, 2, 4 or 8                     */
@@ -92,7 +92,7 @@ typedef struct sar_tuning_t {
                           /*     loads and cached stores, 2 = planned (default).  One launch per     */
                           /*     round plans per row: streaming unless the data is read again within */
                           /*     `reuse_rounds`.  The column executor has one policy per launch: it  */
-                          /*     plans streaming loads when values are forwarded, else all cached    */
+                          /*     plans streaming loads when every re-read is forwarded, else cached  */
     int32_t reuse_rounds; /* look-ahead of policy 2, in rounds                                       */
     int32_t reverse_odd;  /* 1 = odd rounds walk their tiles backwards (keeps the cache tail warm)   */
     int32_t segments;     /* >1: cut every row into this many pieces and run the whole schedule      */
@@ -108,13 +108,13 @@ typedef struct sar_tuning_t {
     int32_t col_forward;  /* column executor: 1 = a value a lane wrote in an earlier round and needs  */
                           /*     again is kept in LDS and not loaded again (all stores still happen; */
                           /*     same bits); 0 = every operand is loaded from its rank buffer        */
-    int32_t col_slots;    /* column executor: most values kept per lane (0 = as many as fit in LDS)  */
+    int32_t col_slots;    /* column executor: most values kept per lane (0 = chosen by the planner)  */
     int32_t col_light_sync; /* column executor: 1 = between rounds the waves of a workgroup only meet   */
                           /*     (no wait for their stores) whenever no lane reads bytes another lane */
                           /*     wrote; 0 = always a full barrier                                     */
-    int32_t col_latency_plan; /* column executor: the plan for few columns (row table copied into LDS, the  */
-                          /*     inputs of the first rows fetched into slots before round 0): 0 = never,  */
-                          /*     1 = when there are at most two columns per compute unit, 2 = always      */
+    int32_t col_latency_plan; /* column executor: the plan for few columns (the workgroups copy the  */
+                          /*     row table into LDS first; no forwarding): 0 = never, 1 = when there */
+                          /*     are at most two columns per compute unit, 2 = always               */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */
