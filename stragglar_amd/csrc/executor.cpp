@@ -55,7 +55,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -68,8 +68,10 @@ struct sar_ctx {
 
     // column plan (tune.executor == 1): the whole main schedule as one launch
     bool column = false;
-    uint32_t* d_round_begin = nullptr;
-    uint32_t col_first_op = 0, col_rounds = 0, col_count = 0, col_grid = 0, col_block = 512, col_slots = 0, col_lane_local = 0, col_staged_rows = 0, col_policy = 0;
+    uint32_t* d_group_begin = nullptr;
+    sar::ColumnComp* d_comps = nullptr;
+    uint32_t col_first_op = 0, col_ncomp = 0, col_items = 0, col_grid = 0, col_block = 512, col_slots = 0, col_lane_local = 0,
+             col_table_rows = 0, col_table_groups = 0, col_policy = 0;
     int cu_count = 0;
 
     std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
@@ -87,8 +89,9 @@ void drop_plan(sar_ctx* c) {
     if (c->graph) { (void)hipGraphDestroy(c->graph); c->graph = nullptr; }
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
-    if (c->d_round_begin) { (void)hipFree(c->d_round_begin); c->d_round_begin = nullptr; }
-    c->column = false; c->col_rounds = c->col_count = c->col_grid = c->col_slots = c->col_staged_rows = c->col_policy = 0;
+    if (c->d_group_begin) { (void)hipFree(c->d_group_begin); c->d_group_begin = nullptr; }
+    if (c->d_comps) { (void)hipFree(c->d_comps); c->d_comps = nullptr; }
+    c->column = false; c->col_ncomp = c->col_items = c->col_grid = c->col_slots = c->col_table_rows = c->col_table_groups = c->col_policy = 0;
     c->prework.clear(); c->rounds.clear(); c->prepared = false;
     c->stats = sar_stats_t{};
 }
@@ -293,13 +296,15 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
 // are busy the value whose next use is furthest away gives way, which is known exactly because the
 // whole schedule is.  Rows get DEVOP_GET0 / GET1 / PUT and their slot numbers.
 struct ColumnPlan {
-    std::vector<uint32_t> round_begin;
+    std::vector<uint32_t> group_begin;       // first row of every group (rows of one component and one round), plus the end
+    std::vector<sar::ColumnComp> comps;
+    uint32_t max_comp_rows = 0, max_comp_groups = 0;
     uint64_t widest_row = 0;
     int block = 512;
     uint32_t nslots = 0;
     uint64_t forwarded_bytes = 0;    // operand bytes taken from value slots instead of memory, per run
     bool lane_local = false;         // every row 16-byte aligned and a whole number of vectors long
-    bool staged = false;             // latency plan: the workgroups copy the row table into LDS first
+    bool staged = false;             // latency plan: a workgroup copies the rows of its component into LDS first
     uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
 };
 
@@ -311,11 +316,10 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
     auto cell_of = [&](int rank, uint64_t byte_off) {
         return rank * cells_per_rank + (int)(chunk_bytes ? std::min<uint64_t>(byte_off / chunk_bytes, (uint64_t)s.parts) : 0);
     };
-    struct ColRow { sar::DevOp d; int c0, c1; };
+    struct ColRow { sar::DevOp d; int c0, c1; uint32_t round; };
     std::vector<ColRow> cr;
-    plan.round_begin.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0;
+    plan.group_begin.clear(); plan.comps.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0;
     for (size_t ri = 0; ri < s.rounds.size(); ++ri) {
-        plan.round_begin.push_back((uint32_t)cr.size());
         for (const sar::Op& op : s.rounds[ri]) {
             if (op.kind == SAR_OP_MREDUCE) return set_error(SAR_ESCHED, "internal: multi-source rows have no column form");
             sar::Range rg = sar::lower_range(s, op, elems);
@@ -333,36 +337,69 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
                 r.d.flags = ((((uintptr_t)r.d.p0 | (uintptr_t)r.d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u;
                 r.c0 = cell_of(op.dst_rank, row_doff + base);
                 r.c1 = cell_of(op.src_rank, row_soff + base);
+                r.round = (uint32_t)ri;
                 plan.widest_row = std::max(plan.widest_row, r.d.bytes);
                 cr.push_back(r);
             }
         }
     }
-    plan.round_begin.push_back((uint32_t)cr.size());
     if (cr.size() > 0x7ffffff0ull) return set_error(SAR_EINVAL, "schedule has too many rows");
     const uint32_t nrows = (uint32_t)cr.size();
     const uint32_t never = 0xffffffffu;
+    const int ncells = c->n * cells_per_rank;
+
+    // Components: rows that (transitively) share a cell.  Rows of different components touch disjoint bytes in
+    // every column, so no order is needed between them; within a component the round order is kept.  For the
+    // four algorithms every row moves a chunk to the same chunk index, and the components are the chunk indices.
+    {
+        std::vector<int> parent((size_t)ncells);
+        for (int i = 0; i < ncells; ++i) parent[(size_t)i] = i;
+        auto find = [&](int x) { while (parent[(size_t)x] != x) { parent[(size_t)x] = parent[(size_t)parent[(size_t)x]]; x = parent[(size_t)x]; } return x; };
+        if (c->tune.col_split) for (const auto& r : cr) { const int a = find(r.c0), b2 = find(r.c1); if (a != b2) parent[(size_t)b2] = a; }
+        std::vector<int> comp_of_root((size_t)ncells, -1);
+        std::vector<std::vector<uint32_t>> members;
+        for (uint32_t i = 0; i < nrows; ++i) {
+            const int root = c->tune.col_split ? find(cr[i].c0) : 0;
+            if (comp_of_root[(size_t)root] < 0) { comp_of_root[(size_t)root] = (int)members.size(); members.emplace_back(); }
+            members[(size_t)comp_of_root[(size_t)root]].push_back(i);
+        }
+        std::vector<ColRow> sorted; sorted.reserve(nrows);
+        for (const auto& m : members) {
+            sar::ColumnComp cc{};
+            cc.group_first = (uint32_t)plan.group_begin.size(); cc.row_first = (uint32_t)sorted.size();
+            uint32_t last_round = never;
+            for (uint32_t i : m) {
+                if (cr[i].round != last_round) { plan.group_begin.push_back((uint32_t)sorted.size()); last_round = cr[i].round; }
+                sorted.push_back(cr[i]);
+            }
+            cc.group_end = (uint32_t)plan.group_begin.size(); cc.row_end = (uint32_t)sorted.size();
+            plan.max_comp_rows = std::max(plan.max_comp_rows, cc.row_end - cc.row_first);
+            plan.max_comp_groups = std::max(plan.max_comp_groups, cc.group_end - cc.group_first);
+            plan.comps.push_back(cc);
+        }
+        plan.group_begin.push_back((uint32_t)sorted.size());
+        cr.swap(sorted);
+    }
 
     // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
     plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512) >= 2048 ? 512 : 256);
 
-    // Latency plan: when the columns are so few that they are all resident at once, time goes into dependent round
-    // trips, not bandwidth, and nobody warms the scalar cache: a row read through scalar loads is a trip to L2.  The
-    // workgroups then copy the row table into LDS first.  Forwarding is left out of it: measured, a row whose
-    // operand comes from a slot is no faster there than one whose operand comes from L2.
+    // Latency plan: when the work items are so few that they are all resident at once, time goes into dependent
+    // round trips, not bandwidth, and nobody warms the scalar cache: a row read through scalar loads is a trip to
+    // L2.  A workgroup then copies the rows of its component into LDS first.
     {
         const int lb = sar::column_latency_block();
         const uint64_t lcols = (plan.widest_row + sar::column_bytes(lb) - 1) / sar::column_bytes(lb);
-        const bool few = c->tune.col_latency_plan == 2 || (c->tune.col_latency_plan == 1 && lcols <= 2u * (uint64_t)std::max(1, c->cu_count));
+        const uint64_t items = lcols * plan.comps.size();
+        const bool few = c->tune.col_latency_plan == 2 || (c->tune.col_latency_plan == 1 && items <= 4u * (uint64_t)std::max(1, c->cu_count));
         if (few && (c->tune.col_block == 0 || c->tune.col_block == lb) &&
-            sar::column_table_bytes(nrows, (uint32_t)plan.round_begin.size() - 1) <= sar::column_lds_budget()) {
+            sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) + sar::column_bytes(lb) <= sar::column_lds_budget()) {
             plan.staged = true;
             plan.block = lb;
         }
     }
 
     // per cell, the rows that touch it, in order; a reducing row reads and writes its cell
-    const int ncells = c->n * cells_per_rank;
     struct Ev { uint32_t row; bool reads, writes; };
     std::vector<std::vector<Ev>> ev((size_t)ncells);
     for (uint32_t i = 0; i < nrows; ++i) {
@@ -453,8 +490,9 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
 
     Forwarding fwd = forward(0);
     bool all_found = false;              // every re-read of the column finds its operand in a slot
-    if (c->tune.col_forward && !plan.staged) {
-        const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, sar::column_lds_budget() / sar::column_bytes(plan.block));
+    if (c->tune.col_forward) {
+        const uint64_t table = plan.staged ? sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) : 0u;
+        const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, (sar::column_lds_budget() - table) / sar::column_bytes(plan.block));
         if (c->tune.col_slots > 0) {
             fwd = forward(std::min<uint32_t>(fit, (uint32_t)c->tune.col_slots));
             all_found = fwd.nslots && fwd.bytes == forward(255u).bytes;
@@ -463,14 +501,15 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
             // unit stay resident, up to 10 half of them.  Measured on MI355X, half occupancy pays when every re-read
             // is then found in a slot (what still goes to memory is the cold inputs and the stores), but not for a
             // part of them; and a plan that finds less than a tenth of the bytes the rows move is not worth the
-            // longer row loop.
+            // longer row loop.  (Component by component few values are alive at a time: one for the StragglAR
+            // tables and ring, four for halving-doubling at n = 8.)
             const uint64_t all = forward(255u).bytes;
             fwd = forward(std::min<uint32_t>(fit, 10u));
             if (fwd.bytes != all) fwd = forward(std::min<uint32_t>(fit, 5u));
             all_found = fwd.nslots && fwd.bytes == all;
             uint64_t moved = 0;                  // algorithmic bytes of the rows
             for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : 3u);
-            if (fwd.bytes * 10u < moved) fwd = forward(0);
+            if (fwd.bytes * 10u < moved) { fwd = forward(0); all_found = false; }
         }
     }
     plan.nslots = fwd.nslots; plan.forwarded_bytes = fwd.bytes;
@@ -491,47 +530,47 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
 }
 
 // Which executor is expected to be faster (executor = 2).  Constants are measurements on MI355X.
-// Column kernel without forwarding: 7.1 algorithmic TB/s when there are columns enough to fill the chip
-// and a column is up to ~128 rows long (n = 8), less for longer columns, whose workgroups drift apart
-// and scatter the access streams (6.4 up to 256 rows, 5.3 beyond).  With forwarding what counts is the
-// bytes that still go to memory: 5.0 TB/s when they are mostly stores (three tenths or more of the
-// operands found in slots), 6.0 otherwise.  A workgroup needs about 0.6 us per row while everything
-// stays cache resident, 0.95 us beyond that; one launch per round moves 6.5 TB/s and costs about 3 us
-// per launch.  With the row table in LDS (latency plan) a row costs 0.32-0.65 us.
-bool column_pays(const sar_ctx* c, size_t column_rows, const ColumnPlan& cp) {
+// Column kernel, bandwidth regime: without forwarding 7.1 algorithmic TB/s while a work item is up to ~128
+// rows long, less for longer items, whose workgroups drift apart and scatter the access streams (6.4 up to
+// 256 rows, 5.3 beyond).  With forwarding what counts is the bytes that still go to memory: 5.0 TB/s when
+// they are mostly stores (three tenths or more of the operands found in slots), 6.0 otherwise.  A workgroup
+// needs about 0.6 us per row of its item while everything stays cache resident, 0.95 us beyond that; with
+// the item's rows in LDS (latency plan) 0.32-0.65 us.  One launch per round moves 6.5 TB/s and costs about
+// 3 us per launch.
+bool column_pays(const sar_ctx* c, const ColumnPlan& cp) {
     const double bytes = (double)c->stats.algorithmic_bytes;
+    const double item_rows = (double)cp.max_comp_rows;
     double est_rounds = 0;
     for (const auto& L : c->rounds) if (L.total_tiles) est_rounds += 3.0 + (double)L.algorithmic_bytes / 6.5e6;
     if (cp.staged) {
-        // latency plan: a row costs a round trip to where its data is (0.32 us while the buffers are tiny, 0.45 us
-        // while they fit the L2s, 0.65 us beyond)
         const double resident_bytes = (double)c->bytes_per_rank * c->n;
         const double per_row_us = resident_bytes <= 262144.0 ? 0.32 : resident_bytes <= 33554432.0 ? 0.45 : 0.65;
-        return 4.0 + std::max((double)column_rows * per_row_us, bytes / 5.5e6) <= est_rounds;
+        return 4.0 + std::max(item_rows * per_row_us, bytes / 5.5e6) <= est_rounds;
     }
     const uint64_t cb = sar::column_bytes(cp.block);
-    const double ncols = (double)((cp.widest_row + cb - 1) / cb);
+    const double items = (double)((cp.widest_row + cb - 1) / cb) * (double)cp.comps.size();
     double wgs_per_cu = 2048.0 / cp.block;
     if (cp.nslots) wgs_per_cu = std::max(1.0, std::min(wgs_per_cu, std::floor(160.0 * 1024.0 / ((double)cp.nslots * (double)cb))));
     const double resident = (double)std::max(1, c->cu_count) * wgs_per_cu;
     const double per_row_us = (double)c->bytes_per_rank * c->n <= 200e6 ? 0.6 : 0.95;
-    const double passes = std::ceil(ncols / resident);
+    const double passes = std::ceil(items / resident);
     double est_stream;
     if (cp.nslots) {
         const double to_memory = std::max(0.0, bytes - (double)cp.forwarded_bytes);
         est_stream = to_memory / ((double)cp.forwarded_bytes >= 0.3 * bytes ? 5.0e6 : 6.0e6);             // bytes per us
     } else {
-        est_stream = bytes / (column_rows <= 128 ? 7.1e6 : column_rows <= 256 ? 6.4e6 : 5.3e6);
+        est_stream = bytes / (item_rows <= 128 ? 7.1e6 : item_rows <= 256 ? 6.4e6 : 5.3e6);
     }
-    const double est_column = std::max(est_stream, (double)column_rows * per_row_us * passes) + 4.0;
+    const double est_column = std::max(est_stream, item_rows * per_row_us * passes) + 4.0;
     return est_column <= est_rounds;
 }
 
 int launch_column_once(sar_ctx* c) {
     sar::ColumnLaunch L{};
-    L.ops = c->d_ops + c->col_first_op; L.round_begin = c->d_round_begin;
-    L.nrounds = c->col_rounds; L.ncols = c->col_count;
-    L.staged_rows = c->col_staged_rows; L.lane_local = c->col_lane_local; L.policy = c->col_policy;
+    L.ops = c->d_ops + c->col_first_op; L.group_begin = c->d_group_begin; L.comps = c->d_comps;
+    L.ncomp = c->col_ncomp; L.nitems = c->col_items;
+    L.table_rows = c->col_table_rows; L.table_groups = c->col_table_groups;
+    L.lane_local = c->col_lane_local; L.policy = c->col_policy;
     SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->col_slots, c->stream, L));
     return SAR_OK;
 }
@@ -561,7 +600,8 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.executor >= 0 && t.executor <= 2) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
            (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024) &&
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
-           (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2;
+           (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
+           (t.col_split == 0 || t.col_split == 1);
 }
 
 }  // namespace
@@ -879,7 +919,7 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
             if ((rc = lower_column(c, main_sched->s, rows, cp)) != SAR_OK) { drop_plan(c); return rc; }
             columnar = rows.size() > col_first;
         }
-        if (columnar && c->tune.executor == 2) columnar = column_pays(c, rows.size() - col_first, cp);
+        if (columnar && c->tune.executor == 2) columnar = column_pays(c, cp);
         want_column = columnar;
     } catch (const std::bad_alloc&) { drop_plan(c); return set_error(SAR_ENOMEM, "out of host memory"); }
     if (!rows.empty()) {
@@ -890,19 +930,23 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     if (!ptrs.empty()) SAR_HIP(hipMemcpy(c->d_ptrs, ptrs.data(), ptrs.size() * sizeof(char*), hipMemcpyHostToDevice));
 
     if (want_column) {
-        SAR_HIP(hipMalloc((void**)&c->d_round_begin, cp.round_begin.size() * sizeof(uint32_t)));
-        SAR_HIP(hipMemcpy(c->d_round_begin, cp.round_begin.data(), cp.round_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        SAR_HIP(hipMalloc((void**)&c->d_group_begin, cp.group_begin.size() * sizeof(uint32_t)));
+        SAR_HIP(hipMemcpy(c->d_group_begin, cp.group_begin.data(), cp.group_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+        SAR_HIP(hipMalloc((void**)&c->d_comps, cp.comps.size() * sizeof(sar::ColumnComp)));
+        SAR_HIP(hipMemcpy(c->d_comps, cp.comps.data(), cp.comps.size() * sizeof(sar::ColumnComp), hipMemcpyHostToDevice));
         c->col_block = (uint32_t)cp.block;
         c->col_slots = cp.nslots;
         c->col_lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
-        c->col_staged_rows = cp.staged ? (uint32_t)(rows.size() - col_first) : 0u;
+        c->col_table_rows = cp.staged ? cp.max_comp_rows : 0u;
+        c->col_table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
         c->col_policy = cp.policy;
         const uint64_t cb = sar::column_bytes(cp.block);
         const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
-        if (ncols > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 columns"); }
-        c->col_first_op = col_first; c->col_rounds = (uint32_t)cp.round_begin.size() - 1; c->col_count = (uint32_t)ncols;
+        const uint64_t items = ncols * cp.comps.size();
+        if (items > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 work items"); }
+        c->col_first_op = col_first; c->col_ncomp = (uint32_t)cp.comps.size(); c->col_items = (uint32_t)items;
         const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
-        c->col_grid = (uint32_t)std::min<uint64_t>(ncols, resident);
+        c->col_grid = (uint32_t)std::min<uint64_t>(items, resident);
         c->column = true;
     }
 

@@ -382,45 +382,54 @@ __device__ __forceinline__ ColRow column_row(const DevOp* __restrict__ ops, cons
 static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offsetof(DevOp, kind) == 24 &&
               offsetof(DevOp, flags) == 28 && offsetof(DevOp, slots) == 52, "column_row reads DevOp by position");
 
-// FWD: value slots in LDS (rows flagged DEVOP_GET* / DEVOP_PUT).  LAT: the plan for few columns -- the row
-// table is copied into LDS first (never together with FWD).  POL: cache policy of the whole launch, 0 = all
+// Rows that share no (rank, chunk) cell never depend on each other, whatever round they sit in.  The host
+// therefore splits the rows into connected components (for all four algorithms: one per chunk index) and a
+// work item is one component for one column: its rows, in round order, cut into groups at the round
+// boundaries (a barrier follows each group).  Items are independent of each other.
+//
+// FWD: value slots in LDS (rows flagged DEVOP_GET* / DEVOP_PUT).  LAT: the plan for few items -- the rows and
+// groups of the item's component are copied into LDS first.  POL: cache policy of the whole launch, 0 = all
 // accesses cached, 1 = streaming (nontemporal) loads and cached stores, 2 = streaming loads and stores.  The
 // policy is a template argument because a flavour picked per row at run time does not survive compilation:
 // the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.
 template <int DT, int BLOCK, bool FWD, bool LAT, int POL>
-__global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ round_begin, ColumnLaunch L) {
+__global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
+                                                        const ColumnComp* __restrict__ comps, ColumnLaunch L) {
     typedef typename Elem<DT>::T T;
-    static_assert(!(FWD && LAT), "the latency plan does not forward");
     constexpr uint64_t col_bytes = (uint64_t)BLOCK * 16u;
     constexpr bool LNT = POL >= 1, SNT = POL == 2;
-    // LDS: LAT: [copy of the row table: staged_rows x 64 B][copy of round_begin]; FWD: the value slots, slot k of
-    // lane t at vector k*BLOCK + t.  A lane only ever touches its own vectors, so the slots need no
-    // synchronisation of their own.
-    // (the two tables come as kernel arguments of their own: only a __restrict__ const parameter lets the
-    // compiler read them through scalar loads)
+    // LDS: LAT: [the component's rows: table_rows x 64 B][its group boundaries: table_groups x 4 B, padded to
+    // 16 B]; then FWD: the value slots, slot k of lane t at vector k*BLOCK + t.  A lane only ever touches its
+    // own slot vectors, so the slots need no synchronisation of their own.
+    // (the tables come as kernel arguments of their own: only a __restrict__ const parameter lets the compiler
+    // read them through scalar loads)
     extern __shared__ __align__(16) char lds_raw[];
-    const u4* table = nullptr;
-    const uint32_t* rbegin = round_begin;
-    if (LAT) {
-        // Few workgroups, nobody to warm the scalar cache: a row read through scalar loads costs a trip to L2
-        // (about half a microsecond) and the rows come one after the other.  Fetch the whole table at once.
-        const uint32_t table_vecs = L.staged_rows * 4u;
-        u4* dst = reinterpret_cast<u4*>(lds_raw);
-        const u4* src = reinterpret_cast<const u4*>(ops);
-        for (uint32_t i = threadIdx.x; i < table_vecs; i += BLOCK) dst[i] = src[i];
-        uint32_t* bdst = reinterpret_cast<uint32_t*>(lds_raw) + table_vecs * 4u;
-        for (uint32_t i = threadIdx.x; i <= L.nrounds; i += BLOCK) bdst[i] = round_begin[i];
-        __syncthreads();
-        table = reinterpret_cast<const u4*>(lds_raw);
-        rbegin = bdst;
-    }
-    f4* const mine = reinterpret_cast<f4*>(lds_raw) + threadIdx.x;
-    for (uint32_t col = blockIdx.x; col < L.ncols; col += gridDim.x) {
+    const uint32_t table_vecs = LAT ? L.table_rows * 4u : 0u, group_vecs = LAT ? (L.table_groups + 3u) / 4u : 0u;
+    const u4* const table = reinterpret_cast<const u4*>(lds_raw);
+    uint32_t* const lgroups = reinterpret_cast<uint32_t*>(lds_raw) + table_vecs * 4u;
+    f4* const mine = reinterpret_cast<f4*>(lds_raw) + table_vecs + group_vecs + threadIdx.x;
+    bool first_item = true;
+    for (uint32_t item = blockIdx.x; item < L.nitems; item += gridDim.x) {
+        const uint32_t comp = item % L.ncomp, col = item / L.ncomp;
+        const ColumnComp C = comps[comp];
+        if (LAT) {
+            // Few workgroups, nobody to warm the scalar cache: a row read through scalar loads costs a trip to
+            // L2 (about half a microsecond) and the rows come one after the other.  Fetch them all at once.
+            if (!first_item) __syncthreads();                    // the previous item is done with the table
+            first_item = false;
+            u4* dst = reinterpret_cast<u4*>(lds_raw);
+            const u4* src = reinterpret_cast<const u4*>(ops + C.row_first);
+            const uint32_t nvec = (C.row_end - C.row_first) * 4u, ngrp = C.group_end - C.group_first + 1u;
+            for (uint32_t i = threadIdx.x; i < nvec; i += BLOCK) dst[i] = src[i];
+            for (uint32_t i = threadIdx.x; i < ngrp; i += BLOCK) lgroups[i] = group_begin[C.group_first + i];
+            __syncthreads();
+        }
         const uint64_t off = (uint64_t)col * col_bytes;
         const uint64_t voff = off + ((uint64_t)threadIdx.x << 4);       // this lane's vector within every row
-        for (uint32_t r = 0; r < L.nrounds; ++r) {
+        for (uint32_t g = C.group_first; g < C.group_end; ++g) {
             uint32_t rb, re;
-            if (LAT) { rb = uniform32(rbegin[r]); re = uniform32(rbegin[r + 1u]); } else { rb = rbegin[r]; re = rbegin[r + 1u]; }
+            if (LAT) { rb = uniform32(lgroups[g - C.group_first]) - C.row_first; re = uniform32(lgroups[g - C.group_first + 1u]) - C.row_first; }
+            else { rb = group_begin[g]; re = group_begin[g + 1u]; }
             for (uint32_t j = rb; j < re; ++j) {
                 const ColRow row = column_row<LAT>(ops, table, j);
                 const uint32_t flags = row.flags, kind = row.kind;
@@ -463,7 +472,7 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                     tile_scalar<DT, BLOCK>(kind, p0, p1, off, len);
                 }
             }
-            // This round's stores are complete before this workgroup's loads of the next round.  (Lanes mostly
+            // This group's stores are complete before this workgroup's loads of the next one.  (Lanes mostly
             // re-read what they wrote themselves, but elements change lanes between aligned and unaligned
             // rows and at partial vectors; measured, the barrier also pays for itself by keeping the waves
             // of a workgroup on the same rows.)  When the host has found that every lane only re-reads bytes
@@ -476,15 +485,15 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
 
 uint64_t column_bytes(int block) { return (uint64_t)block * 16u; }
 uint64_t column_lds_budget() { return 65536u; }
-uint64_t column_table_bytes(uint32_t rows, uint32_t nrounds) { return (uint64_t)rows * sizeof(DevOp) + (((uint64_t)nrounds + 1u + 3u) / 4u) * 16u; }
+uint64_t column_table_bytes(uint32_t rows, uint32_t groups) { return (uint64_t)rows * sizeof(DevOp) + (((uint64_t)groups + 3u) / 4u) * 16u; }
 int column_latency_block() { return 256; }
 
 template <int DT, bool FWD, int POL>
 static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hipStream_t st, const ColumnLaunch& L) {
     switch (block) {
-        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.round_begin, L); break;
-        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL>), dim3(grid), dim3(512), lds, st, L.ops, L.round_begin, L); break;
-        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL>), dim3(grid), dim3(1024), lds, st, L.ops, L.round_begin, L); break;
+        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L); break;
+        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L); break;
+        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -492,8 +501,9 @@ static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hi
 
 template <int DT, int POL>
 static hipError_t launch_column_policy(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
-    if (L.staged_rows) {
-        hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.round_begin, L);
+    if (L.table_rows) {
+        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L);
+        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L);
         return hipGetLastError();
     }
     return fwd ? launch_column_block<DT, true, POL>(block, grid, lds, st, L) : launch_column_block<DT, false, POL>(block, grid, lds, st, L);
@@ -510,10 +520,10 @@ static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, bool 
 }
 
 hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, hipStream_t st, const ColumnLaunch& L) {
-    if (L.ncols == 0 || grid == 0 || L.nrounds == 0) return hipSuccess;
-    const bool lat = L.staged_rows != 0;
-    const uint64_t lds = lat ? column_table_bytes(L.staged_rows, L.nrounds) : (uint64_t)nslots * column_bytes(block);
-    if (nslots > 255u || lds > column_lds_budget() || (lat && (nslots || block != column_latency_block()))) return hipErrorInvalidValue;
+    if (L.nitems == 0 || grid == 0 || L.ncomp == 0) return hipSuccess;
+    const bool lat = L.table_rows != 0;
+    const uint64_t lds = (lat ? column_table_bytes(L.table_rows, L.table_groups) : 0u) + (uint64_t)nslots * column_bytes(block);
+    if (nslots > 255u || lds > column_lds_budget() || (lat && block != column_latency_block())) return hipErrorInvalidValue;
     switch (dtype) {
         case SAR_F32: return launch_column_dt<SAR_F32>(block, grid, (uint32_t)lds, nslots != 0, st, L);
         case SAR_F16: return launch_column_dt<SAR_F16>(block, grid, (uint32_t)lds, nslots != 0, st, L);

@@ -42,23 +42,30 @@ uint64_t mreduce_tile_bytes();
 hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t nops, char* const* ptrs,
                           uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
 // column executor: all rounds of COPY / REDUCE_INTO / XREDUCE rows (each exactly one chunk long) in one
-// launch; a column is column_bytes(block) wide.
+// launch.  The rows are sorted into components (sets of rows that share rank-chunk cells with each other and
+// with no other row); a work item is one component for one column of column_bytes(block) bytes.
+struct ColumnComp {
+    uint32_t group_first, group_end;   // the component's groups (rows of one round each) in group_begin[]
+    uint32_t row_first, row_end;       // = group_begin[group_first], group_begin[group_end]
+};
 struct ColumnLaunch {
-    const DevOp* ops;            // the rows of all rounds
-    const uint32_t* round_begin; // rows of round r are ops[round_begin[r] .. round_begin[r+1])
-    uint32_t nrounds, ncols;
-    uint32_t staged_rows;        // 0, or the total number of rows: latency plan, the workgroup copies the table into
-                                 // LDS first (block = column_latency_block(), no value slots)
+    const DevOp* ops;            // the rows, component by component, in round order within a component
+    const uint32_t* group_begin; // rows of group g are ops[group_begin[g] .. group_begin[g+1])
+    const ColumnComp* comps;
+    uint32_t ncomp, nitems;      // nitems = ncomp * number of columns; item i is component i % ncomp of column i / ncomp
+    uint32_t table_rows;         // 0, or the most rows of a component: latency plan, the workgroup copies the rows and
+    uint32_t table_groups;       // group boundaries (at most table_groups) of its component into LDS first (block =
+                                 // column_latency_block())
     uint32_t lane_local;         // != 0 promises that no lane reads bytes another lane wrote (all rows 16-byte
-                                 // aligned, no partial vectors): rounds are then separated by an execution barrier only
+                                 // aligned, no partial vectors): groups are then separated by an execution barrier only
     uint32_t policy;             // whole launch: 0 = cached accesses, 1 = streaming loads, 2 = streaming loads and stores
 };
 // With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots * column_bytes(block) bytes) and
-// rows flagged DEVOP_GET* take their operands from there instead of memory.  Slots, or the staged table
-// (column_table_bytes), must fit column_lds_budget().
+// rows flagged DEVOP_GET* take their operands from there instead of memory.  Slots plus the staged table
+// (column_table_bytes) must fit column_lds_budget().
 uint64_t column_bytes(int block);
 uint64_t column_lds_budget();
-uint64_t column_table_bytes(uint32_t rows, uint32_t nrounds);
+uint64_t column_table_bytes(uint32_t rows, uint32_t groups);
 int column_latency_block();
 hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, hipStream_t st, const ColumnLaunch& L);
 

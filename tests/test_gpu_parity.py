@@ -214,13 +214,13 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
                   dict(col_forward=1, cache_policy=0), dict(col_forward=1, cache_policy=1, col_light_sync=0),
                   dict(col_forward=1, cache_policy=3), dict(col_forward=0, cache_policy=3),
                   dict(col_forward=1, col_latency_plan=1), dict(col_forward=1, col_latency_plan=2, col_slots=2),
-                  dict(col_forward=0, col_latency_plan=2, cache_policy=1)):
-            # these buffers have few columns: unless a case asks for it, keep the plan for few columns (which does
-            # not forward) out of the way
+                  dict(col_forward=0, col_latency_plan=2, cache_policy=1),
+                  dict(col_forward=1, col_split=0), dict(col_forward=0, col_split=0), dict(col_forward=1, col_split=0, col_latency_plan=2)):
+            # these buffers have few columns: unless a case asks for it, keep the plan for few work items out of the way
             got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(dict(col_latency_plan=0), **dict(t, executor=1)))
             st = gpu_ctx.stats()
             assert st.executor == 1
-            if not t["col_forward"] or t.get("col_latency_plan"):
+            if not t["col_forward"]:
                 assert st.forwarded_bytes == 0 and st.col_slots == 0
             else:
                 assert st.col_slots <= min(t.get("col_slots") or 255, 65536 // (16 * st.col_block))
@@ -247,7 +247,8 @@ def test_latency_plan_on_many_columns(gpu_ctx, sarlib, oracle, alg):
     inputs = make_inputs(n, elems, dtype, seed=33)
     want = run_oracle(oracle, alg, inputs, dtype, read_golden("stragglar_n8_cu.txt") if alg == "stragglar" else None, delay=-1.0)
     for t in (dict(col_latency_plan=2, col_wgs=1), dict(col_latency_plan=2, col_wgs=1, col_block=512),
-              dict(col_latency_plan=2, col_forward=0, cache_policy=3), dict(col_latency_plan=0)):
+              dict(col_latency_plan=2, col_forward=0, cache_policy=3), dict(col_latency_plan=0),
+              dict(col_latency_plan=2, col_split=0, col_wgs=1), dict(col_latency_plan=0, col_split=0)):
         got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, read_golden("stragglar_n8_cu.txt") if alg == "stragglar" else None,
                       delay=-1.0, tuning=dict(t, executor=1))
         for r in range(n):
