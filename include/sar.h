@@ -78,7 +78,7 @@ typedef struct sar_stats_t {
     int32_t executor;              /* executor the main schedule was lowered for: 0 per round, 1 column           */
     int32_t col_block;             /* column executor: threads per workgroup in use (0 otherwise)                 */
     int32_t col_slots;             /* column executor: value slots per lane in use (0 = no forwarding)            */
-    int32_t reserved;
+    int32_t col_components;        /* column executor: independent row components (work items per column)        */
     uint64_t forwarded_bytes;      /* part of algorithmic_bytes that the column executor takes from value slots   */
                                    /* in LDS instead of loading it again from the rank buffers                    */
 } sar_stats_t;

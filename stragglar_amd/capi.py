@@ -40,7 +40,7 @@ class Stats(ctypes.Structure):
     _fields_ = [("algorithmic_bytes", ctypes.c_uint64), ("reference_op_bytes", ctypes.c_uint64),
                 ("prework_bytes", ctypes.c_uint64), ("rounds", ctypes.c_int32), ("launches", ctypes.c_int32),
                 ("ops", ctypes.c_int32), ("uses_graph", ctypes.c_int32), ("executor", ctypes.c_int32),
-                ("col_block", ctypes.c_int32), ("col_slots", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("col_block", ctypes.c_int32), ("col_slots", ctypes.c_int32), ("col_components", ctypes.c_int32),
                 ("forwarded_bytes", ctypes.c_uint64)]
 
 

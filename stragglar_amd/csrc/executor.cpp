@@ -974,6 +974,7 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     st.executor = c->column ? 1 : 0;
     st.col_block = c->column ? (int32_t)c->col_block : 0;
     st.col_slots = c->column ? (int32_t)c->col_slots : 0;
+    st.col_components = c->column ? (int32_t)c->col_ncomp : 0;
     st.forwarded_bytes = c->column ? cp.forwarded_bytes : 0;
     c->stats = st;
     c->prepared = true;
