@@ -1,13 +1,15 @@
-// gfx950 device code of the schedule executor: one batched kernel per
-// schedule round plus the small fill / compare / sleep kernels.
+// gfx950 device code of the schedule executor: the column kernel (a whole
+// schedule in one launch), the round kernel (all rows of one round per
+// launch), the multi-source reduce of the pre-work, and the small fill /
+// compare / sleep kernels.
 //
-// The round kernel replaces, for all rows of a round at once, the reference's
-// "ncclSend/ncclRecv into a temp buffer, then reduce_add<<<ceil(count/256),256>>>"
-// (allreduce_8GPU.cu:29-34 and every call site in :60-874).  It is pure
-// streaming work bound by HBM bandwidth: 16-byte accesses per lane, every
-// wavefront touching 1 KiB of consecutive memory per instruction, U
-// independent vectors in flight per lane and stream, one tile per workgroup so
-// that the hardware dispatcher balances rows of different cost.
+// The data kernels replace the reference's "ncclSend/ncclRecv into a temp
+// buffer, then reduce_add<<<ceil(count/256),256>>>" (allreduce_8GPU.cu:29-34
+// and every call site in :60-874).  They are pure streaming work bound by HBM
+// bandwidth: 16-byte accesses per lane, every wavefront touching 1 KiB of
+// consecutive memory per instruction.  Round kernel: U independent vectors in
+// flight per lane and stream, one tile per workgroup so that the hardware
+// dispatcher balances rows of different cost.  Column kernel: see its section.
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>

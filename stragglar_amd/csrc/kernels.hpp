@@ -8,6 +8,7 @@
 namespace sar {
 
 enum : uint32_t {
+    // cache policy per row, honoured by the round and multi-source kernels (the column kernel has one policy per launch)
     DEVOP_LNT = 1u,    // loads are streaming (nontemporal)
     DEVOP_SNT0 = 2u,   // stores to p0 (or to every MREDUCE destination) are streaming
     DEVOP_SNT1 = 4u,   // stores to p1 are streaming (XREDUCE only)
