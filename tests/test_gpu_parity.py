@@ -112,14 +112,16 @@ def test_config4_shape_n6_nonpow2_with_prework(gpu_ctx, sarlib, oracle, dtype):
         assert_bits_equal(got[r], want[r], "rank %d" % r)
 
 
-@pytest.mark.parametrize("n,table", [(12, "synth_nonpow2_n12.txt"), (16, "synth_pow2_n16.txt"), (32, "synth_pow2_n32.txt")])
+@pytest.mark.parametrize("n,table", [(10, "synth_nonpow2_n10.txt"), (12, "synth_nonpow2_n12.txt"), (14, "synth_nonpow2_n14.txt"),
+                                     (16, "synth_pow2_n16.txt"), (24, "synth_nonpow2_n24.txt"), (32, "synth_pow2_n32.txt")])
 def test_larger_rank_counts(gpu_ctx, sarlib, oracle, n, table):
     nbytes = sarlib.pad_bytes(64 << 10, n)
     inputs = make_inputs(n, nbytes // 4, "f32", seed=n)
-    got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, "f32", read_golden(table), delay=0.0)
     want = run_oracle(oracle, "stragglar", inputs, "f32", read_golden(table), delay=0.0)
-    for r in range(n):
-        assert_bits_equal(got[r], want[r], "n=%d rank %d" % (n, r))
+    for t in (dict(), dict(executor=0), dict(executor=1, col_split=0), dict(executor=1, col_latency_plan=0), dict(executor=1, col_forward=0)):
+        got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, "f32", read_golden(table), delay=0.0, tuning=t)
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "n=%d tuning %r rank %d" % (n, t, r))
     if n == 16:
         for alg in ("ring", "rhd", "direct"):
             g = run_gpu(gpu_ctx, sarlib, alg, n, inputs, "f32", None, delay=0.0)
