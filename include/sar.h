@@ -113,8 +113,8 @@ typedef struct sar_tuning_t {
                           /*     (no wait for their stores) whenever no lane reads bytes another lane */
                           /*     wrote; 0 = always a full barrier                                     */
     int32_t col_latency_plan; /* column executor: the plan for few work items (a workgroup copies the */
-                          /*     rows of its item into LDS first): 0 = never, 1 = when there         */
-                          /*     are at most four work items per compute unit, 2 = always           */
+                          /*     rows of its item into LDS first, one vector per lane): 0 = never, 1 = */
+                          /*     when there are at most eight work items per compute unit, 2 = always */
     int32_t col_split;    /* column executor: 1 = rows that share no rank-chunk cell (for the four   */
                           /*     algorithms: rows of different chunk indices) form work items of     */
                           /*     their own, one per component and column; 0 = one item per column   */

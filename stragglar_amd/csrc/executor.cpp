@@ -382,18 +382,20 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
     }
 
     // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
-    plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512) >= 2048 ? 512 : 256);
+    plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512, false) >= 2048 ? 512 : 256);
 
     // Latency plan: when the work items are so few that they are all resident at once, time goes into dependent
     // round trips, not bandwidth, and nobody warms the scalar cache: a row read through scalar loads is a trip to
-    // L2.  A workgroup then copies the rows of its component into LDS first.
+    // L2.  A workgroup then copies the rows of its component into LDS first, and a lane moves one vector per row
+    // (few items are better spread over more workgroups).  Forwarding is kept only where it takes the loads out of
+    // most rows (see below).
     {
         const int lb = sar::column_latency_block();
-        const uint64_t lcols = (plan.widest_row + sar::column_bytes(lb) - 1) / sar::column_bytes(lb);
+        const uint64_t lcols = (plan.widest_row + sar::column_bytes(lb, false) - 1) / sar::column_bytes(lb, false);
         const uint64_t items = lcols * plan.comps.size();
-        const bool few = c->tune.col_latency_plan == 2 || (c->tune.col_latency_plan == 1 && items <= 4u * (uint64_t)std::max(1, c->cu_count));
+        const bool few = c->tune.col_latency_plan == 2 || (c->tune.col_latency_plan == 1 && items <= 8u * (uint64_t)std::max(1, c->cu_count));
         if (few && (c->tune.col_block == 0 || c->tune.col_block == lb) &&
-            sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) + sar::column_bytes(lb) <= sar::column_lds_budget()) {
+            sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) <= sar::column_lds_budget()) {
             plan.staged = true;
             plan.block = lb;
         }
@@ -492,7 +494,7 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
     bool all_found = false;              // every re-read of the column finds its operand in a slot
     if (c->tune.col_forward) {
         const uint64_t table = plan.staged ? sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) : 0u;
-        const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, (sar::column_lds_budget() - table) / sar::column_bytes(plan.block));
+        const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, (sar::column_lds_budget() - table) / sar::column_bytes(plan.block, !plan.staged));
         if (c->tune.col_slots > 0) {
             fwd = forward(std::min<uint32_t>(fit, (uint32_t)c->tune.col_slots));
             all_found = fwd.nslots && fwd.bytes == forward(255u).bytes;
@@ -510,6 +512,16 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
             uint64_t moved = 0;                  // algorithmic bytes of the rows
             for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : 3u);
             if (fwd.bytes * 10u < moved) { fwd = forward(0); all_found = false; }
+            if (plan.staged && fwd.nslots) {
+                // Latency plan: the buffers sit in L2 and an operand from there arrives about as fast as one from a
+                // slot.  What forwarding buys is rows that load nothing at all (copies of a held value: no round trip
+                // in the chain).  Keep it when two thirds of the rows are such (the broadcast trees of the StragglAR
+                // tables and of direct: n = 32 at 1 MiB per rank 17.8 us against 21.8 us), not for chains whose
+                // rows mostly still load (ring, halving-doubling: 12.9 against 11.7 us at n = 8).
+                uint32_t free_rows = 0;
+                for (uint32_t i = 0; i < nrows; ++i) free_rows += cr[i].d.kind == SAR_OP_COPY && (fwd.flags[i] & sar::DEVOP_GET1);
+                if (free_rows * 3u < nrows * 2u) { fwd = forward(0); all_found = false; }
+            }
         }
     }
     plan.nslots = fwd.nslots; plan.forwarded_bytes = fwd.bytes;
@@ -547,7 +559,7 @@ bool column_pays(const sar_ctx* c, const ColumnPlan& cp) {
         const double per_row_us = resident_bytes <= 262144.0 ? 0.32 : resident_bytes <= 33554432.0 ? 0.45 : 0.65;
         return 4.0 + std::max(item_rows * per_row_us, bytes / 5.5e6) <= est_rounds;
     }
-    const uint64_t cb = sar::column_bytes(cp.block);
+    const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
     const double items = (double)((cp.widest_row + cb - 1) / cb) * (double)cp.comps.size();
     double wgs_per_cu = 2048.0 / cp.block;
     if (cp.nslots) wgs_per_cu = std::max(1.0, std::min(wgs_per_cu, std::floor(160.0 * 1024.0 / ((double)cp.nslots * (double)cb))));
@@ -940,7 +952,7 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
         c->col_table_rows = cp.staged ? cp.max_comp_rows : 0u;
         c->col_table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
         c->col_policy = cp.policy;
-        const uint64_t cb = sar::column_bytes(cp.block);
+        const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
         const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
         const uint64_t items = ncols * cp.comps.size();
         if (items > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 work items"); }

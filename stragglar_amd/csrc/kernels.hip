@@ -398,11 +398,16 @@ template <int DT, int BLOCK, bool FWD, bool LAT, int POL>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
                                                         const ColumnComp* __restrict__ comps, ColumnLaunch L) {
     typedef typename Elem<DT>::T T;
-    constexpr uint64_t col_bytes = (uint64_t)BLOCK * 16u;
+    // Vectors per lane and row: two when values are forwarded in the bandwidth regime (the loads that remain are
+    // few and far between, and two in flight per lane pay: +2 to +9 %), one otherwise (every row loads and
+    // occupancy covers the latency; few items are better spread over more workgroups).
+    constexpr uint32_t V = (FWD && !LAT) ? 2u : 1u;
+    constexpr uint64_t col_bytes = (uint64_t)BLOCK * 16u * V;
     constexpr bool LNT = POL >= 1, SNT = POL == 2;
     // LDS: LAT: [the component's rows: table_rows x 64 B][its group boundaries: table_groups x 4 B, padded to
     // 16 B]; then FWD: the value slots, slot k of lane t at vector k*BLOCK + t.  A lane only ever touches its
-    // own slot vectors, so the slots need no synchronisation of their own.
+    // own slot vectors, so the slots need no synchronisation of their own.  (With V vectors per lane slot k, vector v
+    // of lane t sits at (k*V + v)*BLOCK + t.)
     // (the tables come as kernel arguments of their own: only a __restrict__ const parameter lets the compiler
     // read them through scalar loads)
     extern __shared__ __align__(16) char lds_raw[];
@@ -442,19 +447,34 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                     if (voff + 16u <= bytes) {
                         const uint32_t slots = FWD ? row.slots : 0u;
                         const bool get0 = FWD && (flags & DEVOP_GET0), get1 = FWD && (flags & DEVOP_GET1);
+                        constexpr uint64_t vstep = (uint64_t)BLOCK * 16u;
                         if (FWD && kind == SAR_OP_COPY && get1) {
                             // A copy of a held value is a store and nothing else.  It has a path of its own so
                             // that it does not pass the wait for loaded operands below: the memory counter
                             // runs in order, and that wait would also sit out the stores of the rows before.
-                            st16<SNT>(p0 + voff, mine[(slots >> 8 & 0xffu) * BLOCK]);
+#pragma unroll
+                            for (uint32_t v = 0; v < V; ++v)
+                                if (voff + v * vstep + 16u <= bytes) st16<SNT>(p0 + voff + v * vstep, mine[((slots >> 8 & 0xffu) * V + v) * BLOCK]);
                         } else {
-                            f4 a = {0.f, 0.f, 0.f, 0.f}, b;
-                            if (get1) b = mine[(slots >> 8 & 0xffu) * BLOCK]; else b = ld16<LNT>(p1 + voff);
-                            if (kind != SAR_OP_COPY) { if (get0) a = mine[(slots & 0xffu) * BLOCK]; else a = ld16<LNT>(p0 + voff); }
-                            const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
-                            st16<SNT>(p0 + voff, s);
-                            if (kind == SAR_OP_XREDUCE) st16<SNT>(p1 + voff, s);
-                            if (FWD && (flags & DEVOP_PUT)) mine[(slots >> 16 & 0xffu) * BLOCK] = s;
+                            f4 a[V], b[V];
+#pragma unroll
+                            for (uint32_t v = 0; v < V; ++v) {
+                                a[v] = f4{0.f, 0.f, 0.f, 0.f};
+                                const uint64_t o = voff + v * vstep;
+                                const uint64_t oc = o + 16u <= bytes ? o : voff;          // past the end: reload the first vector, keep nothing
+                                if (get1) b[v] = mine[((slots >> 8 & 0xffu) * V + v) * BLOCK]; else b[v] = ld16<LNT>(p1 + oc);
+                                if (kind != SAR_OP_COPY) { if (get0) a[v] = mine[((slots & 0xffu) * V + v) * BLOCK]; else a[v] = ld16<LNT>(p0 + oc); }
+                            }
+#pragma unroll
+                            for (uint32_t v = 0; v < V; ++v) {
+                                const uint64_t o = voff + v * vstep;
+                                if (o + 16u <= bytes) {
+                                    const f4 s = kind == SAR_OP_COPY ? b[v] : add16<DT>(a[v], b[v]);
+                                    st16<SNT>(p0 + o, s);
+                                    if (kind == SAR_OP_XREDUCE) st16<SNT>(p1 + o, s);
+                                    if (FWD && (flags & DEVOP_PUT)) mine[((slots >> 16 & 0xffu) * V + v) * BLOCK] = s;
+                                }
+                            }
                         }
                     }
                     // the < 16 bytes behind the last whole vector of the row, in the column that holds them
@@ -485,7 +505,7 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
     }
 }
 
-uint64_t column_bytes(int block) { return (uint64_t)block * 16u; }
+uint64_t column_bytes(int block, bool two_vectors) { return (uint64_t)block * 16u * (two_vectors ? 2u : 1u); }
 uint64_t column_lds_budget() { return 65536u; }
 uint64_t column_table_bytes(uint32_t rows, uint32_t groups) { return (uint64_t)rows * sizeof(DevOp) + (((uint64_t)groups + 3u) / 4u) * 16u; }
 int column_latency_block() { return 256; }
@@ -524,7 +544,7 @@ static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, bool 
 hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, hipStream_t st, const ColumnLaunch& L) {
     if (L.nitems == 0 || grid == 0 || L.ncomp == 0) return hipSuccess;
     const bool lat = L.table_rows != 0;
-    const uint64_t lds = (lat ? column_table_bytes(L.table_rows, L.table_groups) : 0u) + (uint64_t)nslots * column_bytes(block);
+    const uint64_t lds = (lat ? column_table_bytes(L.table_rows, L.table_groups) : 0u) + (uint64_t)nslots * column_bytes(block, nslots != 0 && !lat);
     if (nslots > 255u || lds > column_lds_budget() || (lat && block != column_latency_block())) return hipErrorInvalidValue;
     switch (dtype) {
         case SAR_F32: return launch_column_dt<SAR_F32>(block, grid, (uint32_t)lds, nslots != 0, st, L);

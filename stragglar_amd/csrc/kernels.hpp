@@ -44,7 +44,8 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
                           uint32_t total_tiles, uint32_t tiles_per_op, uint32_t interleave, uint32_t reverse);
 // column executor: all rounds of COPY / REDUCE_INTO / XREDUCE rows (each exactly one chunk long) in one
 // launch.  The rows are sorted into components (sets of rows that share rank-chunk cells with each other and
-// with no other row); a work item is one component for one column of column_bytes(block) bytes.
+// with no other row); a work item is one component for one column of column_bytes(block, two_vectors) bytes: one
+// 16-byte vector per lane and row, two with forwarding (nslots > 0) outside the latency plan.
 struct ColumnComp {
     uint32_t group_first, group_end;   // the component's groups (rows of one round each) in group_begin[]
     uint32_t row_first, row_end;       // = group_begin[group_first], group_begin[group_end]
@@ -61,10 +62,10 @@ struct ColumnLaunch {
                                  // aligned, no partial vectors): groups are then separated by an execution barrier only
     uint32_t policy;             // whole launch: 0 = cached accesses, 1 = streaming loads, 2 = streaming loads and stores
 };
-// With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots * column_bytes(block) bytes) and
+// With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots vectors per lane and vector of the row) and
 // rows flagged DEVOP_GET* take their operands from there instead of memory.  Slots plus the staged table
 // (column_table_bytes) must fit column_lds_budget().
-uint64_t column_bytes(int block);
+uint64_t column_bytes(int block, bool two_vectors);
 uint64_t column_lds_budget();
 uint64_t column_table_bytes(uint32_t rows, uint32_t groups);
 int column_latency_block();
