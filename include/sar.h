@@ -252,6 +252,14 @@ int sar_launch_bytes(sar_ctx* ctx, uint64_t* bytes, int cap, int* count);
 int sar_sleep_ticks(sar_ctx* ctx, float delay_ms, int64_t* ticks);
 
 int sar_stats(sar_ctx* ctx, sar_stats_t* out);
+/* What sar_prepare would decide for `n` rank buffers of `bytes_per_rank` bytes, worked out on the host alone: no
+   device, no context, nothing is allocated (launches, executor, column width, components, value slots, forwarded
+   bytes).  `tuning` NULL = the defaults; `compute_units` 0 = 256 (MI355X).  No counterpart in the reference, whose
+   executors are fixed code (allreduce_8GPU.cu:555-874); meant for tools and tests that inspect a plan. */
+/* the tuning a new context starts with (no device needed) */
+int sar_default_tuning(sar_tuning_t* out);
+int sar_plan(const sar_schedule* prework, const sar_schedule* main_schedule, int n, uint64_t bytes_per_rank, int dtype,
+             const sar_tuning_t* tuning, int compute_units, sar_stats_t* out);
 
 #ifdef __cplusplus
 }

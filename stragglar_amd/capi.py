@@ -70,7 +70,7 @@ EXPORTS = [
     "sar_create", "sar_destroy", "sar_alloc_ranks", "sar_adopt_ranks", "sar_upload", "sar_download", "sar_fill_const",
     "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
-    "sar_launch_bytes", "sar_sleep_ticks", "sar_stats",
+    "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_default_tuning",
 ]
 
 
@@ -122,6 +122,8 @@ class Library:
             "sar_launch_bytes": (c_int, [vp, P(u64), c_int, P(c_int)]),
             "sar_sleep_ticks": (c_int, [vp, ctypes.c_float, P(ctypes.c_int64)]),
             "sar_stats": (c_int, [vp, P(Stats)]),
+            "sar_plan": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, P(Stats)]),
+            "sar_default_tuning": (c_int, [P(Tuning)]),
         }
         assert sorted(sig) == sorted(EXPORTS)
         for name, (res, args) in sig.items():
@@ -140,6 +142,24 @@ class Library:
 
     def pad_bytes(self, nbytes: int, n: int) -> int:
         return int(self.lib.sar_pad_bytes(nbytes, n))
+
+    def default_tuning(self) -> "Tuning":
+        t = Tuning()
+        self.check(self.lib.sar_default_tuning(ctypes.byref(t)))
+        return t
+
+    def plan(self, main: "Schedule", n: int, bytes_per_rank: int, dtype: str = "f32", prework: Optional["Schedule"] = None,
+             compute_units: int = 0, **tuning) -> "Stats":
+        """What ``Context.prepare`` would decide, worked out on the host alone (no device needed)."""
+        t = self.default_tuning()
+        for k, v in tuning.items():
+            if not hasattr(t, k):
+                raise KeyError(k)
+            setattr(t, k, v)
+        st = Stats()
+        self.check(self.lib.sar_plan(prework.handle if prework else None, main.handle, n, bytes_per_rank, DTYPES[dtype],
+                                     ctypes.byref(t), compute_units, ctypes.byref(st)))
+        return st
 
     def parse(self, text: str, n: int) -> "Schedule":
         raw = text.encode()

@@ -605,6 +605,45 @@ int launch_all(sar_ctx* c, const std::vector<Launch>& v) {
 
 int launch_main(sar_ctx* c) { return c->column ? launch_column_once(c) : launch_all(c, c->rounds); }
 
+// Everything sar_prepare decides, on the host alone: the rows of both executors, and whether the column executor runs.
+int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, std::vector<sar::DevOp>& rows,
+                 std::vector<char*>& ptrs, ColumnPlan& cp, uint32_t* col_first, bool* want_column) {
+    int rc;
+    *col_first = 0; *want_column = false;
+    try {
+        if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) return rc;
+        if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) return rc;
+        sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &c->stats.algorithmic_bytes, nullptr);
+        bool columnar = c->tune.executor != 0;
+        for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
+        if (columnar) {
+            *col_first = (uint32_t)rows.size();
+            if ((rc = lower_column(c, main_sched->s, rows, cp)) != SAR_OK) return rc;
+            columnar = rows.size() > *col_first;
+        }
+        if (columnar && c->tune.executor == 2) columnar = column_pays(c, cp);
+        *want_column = columnar;
+    } catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory"); }
+    return SAR_OK;
+}
+
+sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column) {
+    sar_stats_t st{};
+    sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
+    if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
+    st.rounds = (int)main_sched->s.rounds.size();
+    for (const auto& r : main_sched->s.rounds) st.ops += (int)r.size();
+    if (column) st.launches += 1;
+    else for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
+    for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
+    st.executor = column ? 1 : 0;
+    st.col_block = column ? (int32_t)cp.block : 0;
+    st.col_slots = column ? (int32_t)cp.nslots : 0;
+    st.col_components = column ? (int32_t)cp.comps.size() : 0;
+    st.forwarded_bytes = column ? cp.forwarded_bytes : 0;
+    return st;
+}
+
 bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 3 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
@@ -919,21 +958,8 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     drop_plan(c);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
     ColumnPlan cp; uint32_t col_first = 0; bool want_column = false;
-    int rc;
-    try {
-        if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) { drop_plan(c); return rc; }
-        if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) { drop_plan(c); return rc; }
-        sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &c->stats.algorithmic_bytes, nullptr);
-        bool columnar = c->tune.executor != 0;
-        for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
-        if (columnar) {
-            col_first = (uint32_t)rows.size();
-            if ((rc = lower_column(c, main_sched->s, rows, cp)) != SAR_OK) { drop_plan(c); return rc; }
-            columnar = rows.size() > col_first;
-        }
-        if (columnar && c->tune.executor == 2) columnar = column_pays(c, cp);
-        want_column = columnar;
-    } catch (const std::bad_alloc&) { drop_plan(c); return set_error(SAR_ENOMEM, "out of host memory"); }
+    int rc = plan_on_host(c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column);
+    if (rc != SAR_OK) { drop_plan(c); return rc; }
     if (!rows.empty()) {
         SAR_HIP(hipMalloc((void**)&c->d_ops, rows.size() * sizeof(sar::DevOp)));
         SAR_HIP(hipMemcpy(c->d_ops, rows.data(), rows.size() * sizeof(sar::DevOp), hipMemcpyHostToDevice));
@@ -962,15 +988,7 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
         c->column = true;
     }
 
-    sar_stats_t st{};
-    sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
-    if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
-    st.rounds = (int)main_sched->s.rounds.size();
-    for (const auto& r : main_sched->s.rounds) st.ops += (int)r.size();
-    if (c->column) st.launches += 1;
-    else for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
-    for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
-
+    sar_stats_t st = plan_stats(c, prework, main_sched, cp, c->column);
     if (use_graph) {
         // the main rounds as one graph: kernel nodes only (no memset nodes)
         hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
@@ -983,11 +1001,6 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
         if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e)); }
         st.uses_graph = 1;
     }
-    st.executor = c->column ? 1 : 0;
-    st.col_block = c->column ? (int32_t)c->col_block : 0;
-    st.col_slots = c->column ? (int32_t)c->col_slots : 0;
-    st.col_components = c->column ? (int32_t)c->col_ncomp : 0;
-    st.forwarded_bytes = c->column ? cp.forwarded_bytes : 0;
     c->stats = st;
     c->prepared = true;
     return SAR_OK;
@@ -1080,6 +1093,40 @@ int sar_stats(sar_ctx* c, sar_stats_t* out) {
     if (!c || !out) return set_error(SAR_EINVAL, "null argument");
     if (!c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
     *out = c->stats; return SAR_OK;
+}
+
+int sar_default_tuning(sar_tuning_t* out) {
+    if (!out) return set_error(SAR_EINVAL, "null argument");
+    *out = sar_ctx().tune; return SAR_OK;
+}
+
+int sar_plan(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+             const sar_tuning_t* tuning, int compute_units, sar_stats_t* out) {
+    if (!main_sched || !out) return set_error(SAR_EINVAL, "null argument");
+    if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
+    if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
+    if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+    if (tuning && !valid_tuning(*tuning)) return set_error(SAR_EINVAL, "tuning value out of range");
+    for (const sar_schedule* s : {prework, main_sched}) {
+        if (!s) continue;
+        if (s->s.n != n) return set_error(SAR_EINVAL, "schedule and rank count disagree");
+        std::string why = sar::validate(s->s);
+        if (!why.empty()) return set_error(SAR_ESCHED, why);
+    }
+    // a context that never touches the device: rank buffers at made-up, suitably aligned addresses (only ever
+    // used for arithmetic here)
+    sar_ctx c;
+    c.n = n; c.dtype = dtype; c.bytes_per_rank = bytes_per_rank;
+    c.cu_count = compute_units > 0 ? compute_units : 256;
+    if (tuning) c.tune = *tuning;
+    const uint64_t stride = (bytes_per_rank + (2u << 20) - 1) & ~(uint64_t)((2u << 20) - 1);
+    for (int r = 0; r < n; ++r) c.adopted.push_back(reinterpret_cast<char*>((uintptr_t)1 << 40) + (uint64_t)r * stride);
+    std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
+    ColumnPlan cp; uint32_t col_first = 0; bool want_column = false;
+    int rc = plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column);
+    if (rc != SAR_OK) return rc;
+    *out = plan_stats(&c, prework, main_sched, cp, want_column);
+    return SAR_OK;
 }
 
 }  // extern "C"

@@ -1,0 +1,113 @@
+"""Host-side planning (sar_plan): what the executor would do for a schedule, checked without a GPU.
+
+The planner decides how rows become work items of the column kernel (components of rows that share
+rank-chunk cells), which operands are forwarded through value slots, and which executor runs.  The counts
+it must arrive at follow from the schedules' structure (allreduce_8GPU.cu:555-874 for the StragglAR table,
+:146-198 ring, :221-532 halving-doubling, :60-113 direct)."""
+import pytest
+
+from conftest import read_golden
+
+MIB = 1 << 20
+
+
+def plan(sarlib, alg, n, nbytes, dtype="f32", table=None, delay=False, **tuning):
+    if alg == "stragglar":
+        main = sarlib.parse(read_golden(table), n) if table else sarlib.builtin("stragglar", n)
+        pre = sarlib.builtin("prework_rs", n) if delay else None
+    else:
+        main = sarlib.builtin(alg, n)
+        pre = sarlib.builtin("prework_ar", n) if (delay and alg == "direct") else None
+    return sarlib.plan(main, n, nbytes, dtype, prework=pre, **tuning)
+
+
+def test_default_tuning_needs_no_device(sarlib):
+    t = sarlib.default_tuning().as_dict()
+    assert t["executor"] == 2 and t["col_forward"] == 1 and t["col_split"] == 1 and t["cache_policy"] == 2
+
+
+@pytest.mark.parametrize("table", ["stragglar_n8_cu.txt", "synth_pow2_n8.txt"])
+def test_stragglar_n8_plan(sarlib, table):
+    S = sarlib.pad_bytes(256 * MIB, 8)
+    st = plan(sarlib, "stragglar", 8, S, table=table)
+    C = S // 7
+    assert st.algorithmic_bytes == 112 * C == 16 * S          # 42 copies + 7 exchanges
+    assert st.reference_op_bytes == 22 * S                    # temp staging + reduce_add as the reference runs them
+    assert (st.rounds, st.ops) == (9, 49)
+    assert st.executor == 1 and st.launches == 1
+    assert st.col_components == 7                             # one per chunk: an exchange and its broadcast tree
+    assert st.col_slots == 1                                  # one value alive per item
+    assert st.forwarded_bytes == 42 * C                       # every re-read
+    assert st.col_block == 512
+    # all rows of a column in round order instead: four values alive at a time
+    st0 = plan(sarlib, "stragglar", 8, S, table=table, col_split=0)
+    assert st0.col_components == 1 and st0.col_slots == 4 and st0.forwarded_bytes == 42 * C
+    # forwarding off, one launch per round
+    assert plan(sarlib, "stragglar", 8, S, table=table, col_forward=0).forwarded_bytes == 0
+    st_r = plan(sarlib, "stragglar", 8, S, table=table, executor=0)
+    assert st_r.executor == 0 and st_r.launches == 9 and st_r.col_components == 0
+
+
+def test_comparators_n8_plan(sarlib):
+    S = sarlib.pad_bytes(256 * MIB, 8)
+    Cn = S // 8
+    ring = plan(sarlib, "ring", 8, S)
+    assert ring.algorithmic_bytes == 35 * S and ring.rounds == 14
+    assert ring.col_components == 8 and ring.col_slots == 1
+    # per chunk: 6 of the 7 reduce-scatter steps read the partial sum of the step before, and all 7 all-gather
+    # steps copy the held result
+    assert ring.forwarded_bytes == 8 * 13 * Cn
+    rhd = plan(sarlib, "rhd", 8, S)
+    assert rhd.algorithmic_bytes == 35 * S and rhd.rounds == 6
+    assert rhd.col_components == 8 and rhd.col_slots == 4     # a butterfly over 8 ranks: 4, 2, 1 partial sums alive
+    assert rhd.forwarded_bytes == 8 * (6 + 7) * Cn            # reduce tree: 4 + 2 operands of the later steps; 7 copies
+    direct = plan(sarlib, "direct", 8, S)
+    assert direct.algorithmic_bytes == 16 * S and direct.rounds == 3     # the exchange, then 2 + 4 copies
+    assert direct.col_components == 1 and direct.col_slots == 1 and direct.forwarded_bytes == 6 * S
+    for st in (ring, rhd, direct):
+        assert st.executor == 1 and st.launches == 1
+
+
+@pytest.mark.parametrize("n,table", [(4, "stragglar_n4_cu.txt"), (6, "synth_nonpow2_n6.txt"), (12, "synth_nonpow2_n12.txt"),
+                                     (16, "synth_pow2_n16.txt"), (24, "synth_nonpow2_n24.txt"), (32, "synth_pow2_n32.txt")])
+def test_stragglar_tables_split_into_one_item_per_chunk(sarlib, n, table):
+    S = sarlib.pad_bytes(64 * MIB, n)
+    st = plan(sarlib, "stragglar", n, S, table=table)
+    C = S // (n - 1)
+    assert st.col_components == n - 1 and st.col_slots == 1
+    assert st.forwarded_bytes == (n - 1) * (n - 2) * C        # every rank but the two of the exchange copies the chunk once
+    assert st.algorithmic_bytes == (n - 1) * (4 + 2 * (n - 2)) * C
+
+
+def test_small_messages_take_the_plan_for_few_items(sarlib):
+    S = sarlib.pad_bytes(4096, 8)
+    st = plan(sarlib, "stragglar", 8, S)
+    assert st.executor == 1 and st.launches == 1 and st.col_block == 256 and st.col_components == 7
+    assert st.col_slots == 1                                  # broadcast trees keep forwarding there
+    ring = plan(sarlib, "ring", 8, S)
+    assert ring.executor == 1 and ring.col_slots == 0         # chains whose rows mostly still load do not
+    assert plan(sarlib, "ring", 8, S, col_latency_plan=0).col_slots == 1
+
+
+def test_prework_and_misaligned_buffers(sarlib):
+    S = sarlib.pad_bytes(16 * MIB, 8)
+    st = plan(sarlib, "stragglar", 8, S, delay=True)
+    assert st.prework_bytes == 8 * S and st.launches == 2     # one multi-source launch, then the column kernel
+    # chunk of 4k+2 elements: rows keep their alignment only where the chunk offset happens to allow it
+    odd = plan(sarlib, "stragglar", 8, 7 * 4 * 1026, col_latency_plan=0)
+    assert 0 <= odd.forwarded_bytes < 42 * 4 * 1026
+    # a schedule with multi-source rows as the main schedule runs one launch per round
+    pre = sarlib.builtin("prework_rs", 8)
+    assert sarlib.plan(pre, 8, S).executor == 0
+
+
+def test_plan_argument_checks(sarlib):
+    main = sarlib.builtin("ring", 8)
+    with pytest.raises(Exception):
+        sarlib.plan(main, 4, 1 << 20)                         # rank count of the schedule
+    with pytest.raises(Exception):
+        sarlib.plan(main, 8, 0)
+    with pytest.raises(Exception):
+        sarlib.plan(main, 8, 1 << 20, col_block=333)
+    with pytest.raises(KeyError):
+        sarlib.plan(main, 8, 1 << 20, no_such_knob=1)
