@@ -173,6 +173,10 @@ def main():
                 "kernel": "sar::column_kernel<f32, %d, %s>" % (st.col_block, "forwarding" if st.col_slots else "no forwarding") if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
                 "launches": len(launch_bytes),
                 "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
+    if st.forwarded_bytes:
+        roofline["note"] = ("frac can pass 1: %.1f %% of the algorithmic bytes are re-reads of values the same lane wrote, served from LDS; "
+                            "the memory side (traffic) ran at %.0f GB/s" % (100.0 * st.forwarded_bytes / st.algorithmic_bytes,
+                                                                          (mean_launch_bytes - st.forwarded_bytes / len(launch_bytes)) / mean_launch_ms / 1e6))
     # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
     rec = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
