@@ -81,6 +81,8 @@ typedef struct sar_stats_t {
     int32_t col_components;        /* column executor: independent row components (work items per column)        */
     uint64_t forwarded_bytes;      /* part of algorithmic_bytes that the column executor takes from value slots   */
                                    /* in LDS instead of loading it again from the rank buffers                    */
+    int32_t fused_prework;         /* 1 if sar_run(delay 0) runs pre-work + main schedule as a single launch      */
+    int32_t reserved;
 } sar_stats_t;
 
 /* run-time tunables of the executors; sar_get_tuning() reports the defaults */
@@ -119,6 +121,10 @@ typedef struct sar_tuning_t {
                           /*     algorithms: rows of different chunk indices) form work items of     */
                           /*     their own, one per component and column; 0 = one item per column   */
                           /*     walks all rows in round order                                       */
+    int32_t col_fuse_prework; /* column executor: 1 = sar_run with delay 0 runs pre-work and main     */
+                          /*     schedule as one launch (the pre-work's result for a chunk goes to   */
+                          /*     that chunk's exchange in a value slot); with a delay the pre-work   */
+                          /*     stays a launch of its own, overlapping the straggler's absence      */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

@@ -42,6 +42,14 @@ int elem_size_of(int dtype) { return dtype == SAR_F32 ? 4 : 2; }
 
 }  // namespace
 
+// A column plan as it sits on the device.
+struct ColumnDevice {
+    bool ready = false;
+    uint32_t* d_group_begin = nullptr;
+    sar::ColumnComp* d_comps = nullptr;
+    uint32_t first_op = 0, ncomp = 0, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0;
+};
+
 struct sar_ctx {
     int device = 0;
     hipStream_t stream = nullptr, straggler_stream = nullptr;
@@ -55,7 +63,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -68,10 +76,8 @@ struct sar_ctx {
 
     // column plan (tune.executor == 1): the whole main schedule as one launch
     bool column = false;
-    uint32_t* d_group_begin = nullptr;
-    sar::ColumnComp* d_comps = nullptr;
-    uint32_t col_first_op = 0, col_ncomp = 0, col_items = 0, col_grid = 0, col_block = 512, col_slots = 0, col_lane_local = 0,
-             col_table_rows = 0, col_table_groups = 0, col_policy = 0;
+    ColumnDevice col;                  // the main schedule
+    ColumnDevice fused;                // pre-work + main schedule in one launch (used by sar_run with no delay)
     int cu_count = 0;
 
     std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
@@ -89,9 +95,12 @@ void drop_plan(sar_ctx* c) {
     if (c->graph) { (void)hipGraphDestroy(c->graph); c->graph = nullptr; }
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
-    if (c->d_group_begin) { (void)hipFree(c->d_group_begin); c->d_group_begin = nullptr; }
-    if (c->d_comps) { (void)hipFree(c->d_comps); c->d_comps = nullptr; }
-    c->column = false; c->col_ncomp = c->col_items = c->col_grid = c->col_slots = c->col_table_rows = c->col_table_groups = c->col_policy = 0;
+    for (ColumnDevice* d : {&c->col, &c->fused}) {
+        if (d->d_group_begin) (void)hipFree(d->d_group_begin);
+        if (d->d_comps) (void)hipFree(d->d_comps);
+        *d = ColumnDevice{};
+    }
+    c->column = false;
     c->prework.clear(); c->rounds.clear(); c->prepared = false;
     c->stats = sar_stats_t{};
 }
@@ -306,9 +315,14 @@ struct ColumnPlan {
     bool lane_local = false;         // every row 16-byte aligned and a whole number of vectors long
     bool staged = false;             // latency plan: a workgroup copies the rows of its component into LDS first
     uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
+    bool unsupported = false;        // the rows cannot all run in the column kernel
 };
 
-int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, ColumnPlan& plan) {
+// `scheds`: the schedules to run back to back in the one launch (the main schedule, or pre-work + main); they share
+// `parts`.  Multi-source rows (pre-work) are only taken when every pointer is 16-byte aligned and the row is a whole
+// number of vectors long; otherwise plan.unsupported is set and the caller keeps the pre-work as launches of its own.
+int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, std::vector<sar::DevOp>& rows, std::vector<char*>& ptrs, ColumnPlan& plan) {
+    const sar::Schedule& s = *scheds.back();
     const int es = elem_size_of(c->dtype);
     const uint64_t elems = c->elems();
     const uint64_t chunk_bytes = (elems / (uint64_t)s.parts) * es;
@@ -316,13 +330,15 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
     auto cell_of = [&](int rank, uint64_t byte_off) {
         return rank * cells_per_rank + (int)(chunk_bytes ? std::min<uint64_t>(byte_off / chunk_bytes, (uint64_t)s.parts) : 0);
     };
-    struct ColRow { sar::DevOp d; int c0, c1; uint32_t round; };
+    struct ColRow { sar::DevOp d; int c0, c1; uint32_t round; std::vector<int> mreads, mwrites; };   // m*: cells of a multi-source row
     std::vector<ColRow> cr;
-    plan.group_begin.clear(); plan.comps.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0;
-    for (size_t ri = 0; ri < s.rounds.size(); ++ri) {
-        for (const sar::Op& op : s.rounds[ri]) {
-            if (op.kind == SAR_OP_MREDUCE) return set_error(SAR_ESCHED, "internal: multi-source rows have no column form");
-            sar::Range rg = sar::lower_range(s, op, elems);
+    plan.group_begin.clear(); plan.comps.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0; plan.unsupported = false;
+    uint32_t round_no = 0;
+    for (const sar::Schedule* sp : scheds) {
+      if (sp->parts != s.parts) { plan.unsupported = true; return SAR_OK; }
+      for (size_t ri = 0; ri < sp->rounds.size(); ++ri, ++round_no) {
+        for (const sar::Op& op : sp->rounds[ri]) {
+            sar::Range rg = sar::lower_range(*sp, op, elems);
             const uint64_t row_bytes = rg.len * es;
             if (row_bytes == 0) continue;
             const uint64_t row_doff = rg.dst_off * es, row_soff = rg.src_off * es;
@@ -332,16 +348,32 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
                 ColRow r{};
                 r.d.kind = (uint32_t)op.kind;
                 r.d.bytes = (j == op.nchunks - 1) ? row_bytes - base : chunk_bytes;     // a to_end row ends with a longer chunk
-                r.d.p0 = c->rank_base(op.dst_rank) + row_doff + base;
-                r.d.p1 = c->rank_base(op.src_rank) + row_soff + base;
-                r.d.flags = ((((uintptr_t)r.d.p0 | (uintptr_t)r.d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u;
-                r.c0 = cell_of(op.dst_rank, row_doff + base);
-                r.c1 = cell_of(op.src_rank, row_soff + base);
-                r.round = (uint32_t)ri;
+                r.round = round_no;
+                if (op.kind == SAR_OP_MREDUCE) {
+                    // ring order over the group: x_{r+1}, x_{r+2}, ..., x_{r-1}, x_r (the owner last), as one launch per round has it
+                    const uint64_t off = row_doff + base;
+                    r.d.ptr_off = (uint32_t)ptrs.size(); r.d.nsrc = (uint32_t)op.group;
+                    for (int q = 1; q <= op.group; ++q) { const int rank = (op.dst_rank + q) % op.group; ptrs.push_back(c->rank_base(rank) + off); r.mreads.push_back(cell_of(rank, off)); }
+                    if (op.bcast) { r.d.ndst = (uint32_t)op.group; for (int q = 0; q < op.group; ++q) { ptrs.push_back(c->rank_base(q) + off); r.mwrites.push_back(cell_of(q, off)); } }
+                    else { r.d.ndst = 1; ptrs.push_back(c->rank_base(op.dst_rank) + off); r.mwrites.push_back(cell_of(op.dst_rank, off)); }
+                    bool aligned = (r.d.bytes & 15u) == 0;
+                    for (size_t k = r.d.ptr_off; k < ptrs.size(); ++k) aligned &= ((uintptr_t)ptrs[k] & 15u) == 0;
+                    if (!aligned) { plan.unsupported = true; return SAR_OK; }
+                    r.d.flags = sar::DEVOP_VEC;
+                    r.d.p0 = ptrs[r.d.ptr_off + r.d.nsrc]; r.d.p1 = ptrs[r.d.ptr_off];
+                    r.c0 = r.mwrites[0]; r.c1 = r.mreads[0];
+                } else {
+                    r.d.p0 = c->rank_base(op.dst_rank) + row_doff + base;
+                    r.d.p1 = c->rank_base(op.src_rank) + row_soff + base;
+                    r.d.flags = ((((uintptr_t)r.d.p0 | (uintptr_t)r.d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u;
+                    r.c0 = cell_of(op.dst_rank, row_doff + base);
+                    r.c1 = cell_of(op.src_rank, row_soff + base);
+                }
                 plan.widest_row = std::max(plan.widest_row, r.d.bytes);
                 cr.push_back(r);
             }
         }
+      }
     }
     if (cr.size() > 0x7ffffff0ull) return set_error(SAR_EINVAL, "schedule has too many rows");
     const uint32_t nrows = (uint32_t)cr.size();
@@ -355,7 +387,12 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
         std::vector<int> parent((size_t)ncells);
         for (int i = 0; i < ncells; ++i) parent[(size_t)i] = i;
         auto find = [&](int x) { while (parent[(size_t)x] != x) { parent[(size_t)x] = parent[(size_t)parent[(size_t)x]]; x = parent[(size_t)x]; } return x; };
-        if (c->tune.col_split) for (const auto& r : cr) { const int a = find(r.c0), b2 = find(r.c1); if (a != b2) parent[(size_t)b2] = a; }
+        auto unite = [&](int x, int y) { const int a = find(x), b2 = find(y); if (a != b2) parent[(size_t)b2] = a; };
+        if (c->tune.col_split) for (const auto& r : cr) {
+            unite(r.c0, r.c1);
+            for (int cell : r.mreads) unite(r.c0, cell);
+            for (int cell : r.mwrites) unite(r.c0, cell);
+        }
         std::vector<int> comp_of_root((size_t)ncells, -1);
         std::vector<std::vector<uint32_t>> members;
         for (uint32_t i = 0; i < nrows; ++i) {
@@ -405,6 +442,13 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
     struct Ev { uint32_t row; bool reads, writes; };
     std::vector<std::vector<Ev>> ev((size_t)ncells);
     for (uint32_t i = 0; i < nrows; ++i) {
+        if (cr[i].d.kind == SAR_OP_MREDUCE) {
+            for (int cell : cr[i].mreads)
+                ev[(size_t)cell].push_back({i, true, std::find(cr[i].mwrites.begin(), cr[i].mwrites.end(), cell) != cr[i].mwrites.end()});
+            for (int cell : cr[i].mwrites)
+                if (std::find(cr[i].mreads.begin(), cr[i].mreads.end(), cell) == cr[i].mreads.end()) ev[(size_t)cell].push_back({i, false, true});
+            continue;
+        }
         const bool reduce = cr[i].d.kind != SAR_OP_COPY, both = cr[i].d.kind == SAR_OP_XREDUCE;
         ev[(size_t)cr[i].c0].push_back({i, reduce, true});
         if (cr[i].c1 != cr[i].c0) ev[(size_t)cr[i].c1].push_back({i, true, both});
@@ -459,6 +503,19 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
         };
         for (uint32_t i = 0; i < nrows; ++i) {
             const sar::DevOp& d = cr[i].d;
+            if (d.kind == SAR_OP_MREDUCE) {
+                // all operands come from memory (they are inputs nobody has touched); the result is a new value
+                uint32_t nu = never;
+                for (int cell : cr[i].mwrites) { drop_cell(cell); nu = std::min(nu, next_read(cell, i)); }
+                const int k = nu == never ? -1 : take_slot(nu, i);
+                if (k >= 0) {
+                    slot[(size_t)k].bytes = d.bytes;
+                    for (int cell : cr[i].mwrites) { slot[(size_t)k].cells.push_back(cell); cell_slot[(size_t)cell] = k; }
+                    f.flags[i] |= sar::DEVOP_PUT; f.slots[i] |= (uint32_t)k << 16;
+                    f.nslots = std::max(f.nslots, (uint32_t)k + 1);
+                }
+                continue;
+            }
             const int c0 = cr[i].c0, c1 = cr[i].c1;
             const bool reduce = d.kind != SAR_OP_COPY;
             const bool can = (d.flags & sar::DEVOP_VEC) && c0 != c1;
@@ -510,7 +567,7 @@ int lower_column(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& ro
             if (fwd.bytes != all) fwd = forward(std::min<uint32_t>(fit, 5u));
             all_found = fwd.nslots && fwd.bytes == all;
             uint64_t moved = 0;                  // algorithmic bytes of the rows
-            for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : 3u);
+            for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : r.d.kind == SAR_OP_MREDUCE ? r.d.nsrc + r.d.ndst : 3u);
             if (fwd.bytes * 10u < moved) { fwd = forward(0); all_found = false; }
             if (plan.staged && fwd.nslots) {
                 // Latency plan: the buffers sit in L2 and an operand from there arrives about as fast as one from a
@@ -577,13 +634,36 @@ bool column_pays(const sar_ctx* c, const ColumnPlan& cp) {
     return est_column <= est_rounds;
 }
 
-int launch_column_once(sar_ctx* c) {
+int launch_column_plan(sar_ctx* c, const ColumnDevice& d) {
     sar::ColumnLaunch L{};
-    L.ops = c->d_ops + c->col_first_op; L.group_begin = c->d_group_begin; L.comps = c->d_comps;
-    L.ncomp = c->col_ncomp; L.nitems = c->col_items;
-    L.table_rows = c->col_table_rows; L.table_groups = c->col_table_groups;
-    L.lane_local = c->col_lane_local; L.policy = c->col_policy;
-    SAR_HIP(sar::launch_column(c->dtype, c->col_block, c->col_grid, c->col_slots, c->stream, L));
+    L.ops = c->d_ops + d.first_op; L.group_begin = d.d_group_begin; L.comps = d.d_comps; L.ptrs = c->d_ptrs;
+    L.ncomp = d.ncomp; L.nitems = d.items;
+    L.table_rows = d.table_rows; L.table_groups = d.table_groups;
+    L.lane_local = d.lane_local; L.policy = d.policy;
+    SAR_HIP(sar::launch_column(c->dtype, (int)d.block, d.grid, d.slots, c->stream, L));
+    return SAR_OK;
+}
+
+// Copy a column plan's tables to the device (its rows are in d_ops from `first_op` on).
+int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, ColumnDevice& d) {
+    const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
+    const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
+    const uint64_t items = ncols * cp.comps.size();
+    if (items > 0x7fffffffull) return set_error(SAR_EINVAL, "schedule needs more than 2^31 work items");
+    SAR_HIP(hipMalloc((void**)&d.d_group_begin, cp.group_begin.size() * sizeof(uint32_t)));
+    SAR_HIP(hipMemcpy(d.d_group_begin, cp.group_begin.data(), cp.group_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+    SAR_HIP(hipMalloc((void**)&d.d_comps, cp.comps.size() * sizeof(sar::ColumnComp)));
+    SAR_HIP(hipMemcpy(d.d_comps, cp.comps.data(), cp.comps.size() * sizeof(sar::ColumnComp), hipMemcpyHostToDevice));
+    d.block = (uint32_t)cp.block;
+    d.slots = cp.nslots;
+    d.lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
+    d.table_rows = cp.staged ? cp.max_comp_rows : 0u;
+    d.table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
+    d.policy = cp.policy;
+    d.first_op = first_op; d.ncomp = (uint32_t)cp.comps.size(); d.items = (uint32_t)items;
+    const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
+    d.grid = (uint32_t)std::min<uint64_t>(items, resident);
+    d.ready = true;
     return SAR_OK;
 }
 
@@ -603,13 +683,14 @@ int launch_all(sar_ctx* c, const std::vector<Launch>& v) {
     return SAR_OK;
 }
 
-int launch_main(sar_ctx* c) { return c->column ? launch_column_once(c) : launch_all(c, c->rounds); }
+int launch_main(sar_ctx* c) { return c->column ? launch_column_plan(c, c->col) : launch_all(c, c->rounds); }
 
 // Everything sar_prepare decides, on the host alone: the rows of both executors, and whether the column executor runs.
 int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, std::vector<sar::DevOp>& rows,
-                 std::vector<char*>& ptrs, ColumnPlan& cp, uint32_t* col_first, bool* want_column) {
+                 std::vector<char*>& ptrs, ColumnPlan& cp, uint32_t* col_first, bool* want_column,
+                 ColumnPlan& fused, uint32_t* fused_first, bool* want_fused) {
     int rc;
-    *col_first = 0; *want_column = false;
+    *col_first = 0; *want_column = false; *fused_first = 0; *want_fused = false;
     try {
         if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) return rc;
         if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) return rc;
@@ -618,16 +699,23 @@ int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* ma
         for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
         if (columnar) {
             *col_first = (uint32_t)rows.size();
-            if ((rc = lower_column(c, main_sched->s, rows, cp)) != SAR_OK) return rc;
-            columnar = rows.size() > *col_first;
+            if ((rc = lower_column(c, {&main_sched->s}, rows, ptrs, cp)) != SAR_OK) return rc;
+            columnar = rows.size() > *col_first && !cp.unsupported;
         }
         if (columnar && c->tune.executor == 2) columnar = column_pays(c, cp);
         *want_column = columnar;
+        // Pre-work and main schedule as ONE launch, for runs in which nobody is late (the pre-work then simply
+        // precedes the schedule): its result for a chunk is handed to the exchange of that chunk in a value slot.
+        if (columnar && prework && c->tune.col_fuse_prework) {
+            *fused_first = (uint32_t)rows.size();
+            if ((rc = lower_column(c, {&prework->s, &main_sched->s}, rows, ptrs, fused)) != SAR_OK) return rc;
+            *want_fused = rows.size() > *fused_first && !fused.unsupported;
+        }
     } catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory"); }
     return SAR_OK;
 }
 
-sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column) {
+sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column, bool fused) {
     sar_stats_t st{};
     sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
     if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
@@ -641,6 +729,7 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     st.col_slots = column ? (int32_t)cp.nslots : 0;
     st.col_components = column ? (int32_t)cp.comps.size() : 0;
     st.forwarded_bytes = column ? cp.forwarded_bytes : 0;
+    st.fused_prework = fused ? 1 : 0;
     return st;
 }
 
@@ -652,7 +741,7 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024) &&
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
-           (t.col_split == 0 || t.col_split == 1);
+           (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1);
 }
 
 }  // namespace
@@ -957,8 +1046,8 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_plan(c);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    ColumnPlan cp; uint32_t col_first = 0; bool want_column = false;
-    int rc = plan_on_host(c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column);
+    ColumnPlan cp, fp; uint32_t col_first = 0, fused_first = 0; bool want_column = false, want_fused = false;
+    int rc = plan_on_host(c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused);
     if (rc != SAR_OK) { drop_plan(c); return rc; }
     if (!rows.empty()) {
         SAR_HIP(hipMalloc((void**)&c->d_ops, rows.size() * sizeof(sar::DevOp)));
@@ -968,27 +1057,12 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     if (!ptrs.empty()) SAR_HIP(hipMemcpy(c->d_ptrs, ptrs.data(), ptrs.size() * sizeof(char*), hipMemcpyHostToDevice));
 
     if (want_column) {
-        SAR_HIP(hipMalloc((void**)&c->d_group_begin, cp.group_begin.size() * sizeof(uint32_t)));
-        SAR_HIP(hipMemcpy(c->d_group_begin, cp.group_begin.data(), cp.group_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
-        SAR_HIP(hipMalloc((void**)&c->d_comps, cp.comps.size() * sizeof(sar::ColumnComp)));
-        SAR_HIP(hipMemcpy(c->d_comps, cp.comps.data(), cp.comps.size() * sizeof(sar::ColumnComp), hipMemcpyHostToDevice));
-        c->col_block = (uint32_t)cp.block;
-        c->col_slots = cp.nslots;
-        c->col_lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
-        c->col_table_rows = cp.staged ? cp.max_comp_rows : 0u;
-        c->col_table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
-        c->col_policy = cp.policy;
-        const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
-        const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
-        const uint64_t items = ncols * cp.comps.size();
-        if (items > 0x7fffffffull) { drop_plan(c); return set_error(SAR_EINVAL, "schedule needs more than 2^31 work items"); }
-        c->col_first_op = col_first; c->col_ncomp = (uint32_t)cp.comps.size(); c->col_items = (uint32_t)items;
-        const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
-        c->col_grid = (uint32_t)std::min<uint64_t>(items, resident);
+        if ((rc = upload_column_plan(c, cp, col_first, c->col)) != SAR_OK) { drop_plan(c); return rc; }
         c->column = true;
+        if (want_fused && (rc = upload_column_plan(c, fp, fused_first, c->fused)) != SAR_OK) { drop_plan(c); return rc; }
     }
 
-    sar_stats_t st = plan_stats(c, prework, main_sched, cp, c->column);
+    sar_stats_t st = plan_stats(c, prework, main_sched, cp, c->column, c->fused.ready);
     if (use_graph) {
         // the main rounds as one graph: kernel nodes only (no memset nodes)
         hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
@@ -1011,7 +1085,12 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     if (!(delay_ms <= kMaxDelayMs)) return set_error(SAR_EINVAL, "delay out of range");
     SAR_HIP(hipSetDevice(c->device));
     SAR_HIP(hipEventRecord(c->ev_start, c->stream));
-    if (delay_ms == 0) {
+    bool main_done = false;
+    if (delay_ms == 0 && c->fused.ready && !c->graph_exec) {
+        // nobody is late: pre-work and schedule as the one launch planned for this case
+        int rc = launch_column_plan(c, c->fused); if (rc) return rc;
+        main_done = true;
+    } else if (delay_ms == 0) {
         // nobody is late: pre-work, then the schedule, on one stream
         int rc = launch_all(c, c->prework); if (rc) return rc;
     } else if (delay_ms > 0) {
@@ -1023,7 +1102,8 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
         int rc = launch_all(c, c->prework); if (rc) return rc;
         SAR_HIP(hipStreamWaitEvent(c->stream, c->ev_join, 0));
     }
-    if (c->graph_exec) SAR_HIP(hipGraphLaunch(c->graph_exec, c->stream));
+    if (main_done) {}
+    else if (c->graph_exec) SAR_HIP(hipGraphLaunch(c->graph_exec, c->stream));
     else { int rc = launch_main(c); if (rc) return rc; }
     SAR_HIP(hipEventRecord(c->ev_stop, c->stream));
     SAR_HIP(hipEventSynchronize(c->ev_stop));
@@ -1041,7 +1121,7 @@ int sar_run_profiled(sar_ctx* c, float* ms, int cap, int* count) {
     if (c->column) {
         while (c->ev_prof.size() < 2) { hipEvent_t e; SAR_HIP(hipEventCreate(&e)); c->ev_prof.push_back(e); }
         SAR_HIP(hipEventRecord(c->ev_prof[0], c->stream));
-        int rc = launch_column_once(c); if (rc) return rc;
+        int rc = launch_column_plan(c, c->col); if (rc) return rc;
         SAR_HIP(hipEventRecord(c->ev_prof[1], c->stream));
         SAR_HIP(hipStreamSynchronize(c->stream));
         if (cap > 0) SAR_HIP(hipEventElapsedTime(&ms[0], c->ev_prof[0], c->ev_prof[1]));
@@ -1122,10 +1202,10 @@ int sar_plan(const sar_schedule* prework, const sar_schedule* main_sched, int n,
     const uint64_t stride = (bytes_per_rank + (2u << 20) - 1) & ~(uint64_t)((2u << 20) - 1);
     for (int r = 0; r < n; ++r) c.adopted.push_back(reinterpret_cast<char*>((uintptr_t)1 << 40) + (uint64_t)r * stride);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    ColumnPlan cp; uint32_t col_first = 0; bool want_column = false;
-    int rc = plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column);
+    ColumnPlan cp, fp; uint32_t col_first = 0, fused_first = 0; bool want_column = false, want_fused = false;
+    int rc = plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused);
     if (rc != SAR_OK) return rc;
-    *out = plan_stats(&c, prework, main_sched, cp, want_column);
+    *out = plan_stats(&c, prework, main_sched, cp, want_column, want_column && want_fused);
     return SAR_OK;
 }
 

@@ -360,7 +360,7 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // several rows or several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
 
 // One row as the column kernel uses it, every field wave-uniform (SGPRs).
-struct ColRow { char* p0; char* p1; uint64_t bytes; uint32_t kind, flags, slots; };
+struct ColRow { char* p0; char* p1; uint64_t bytes; uint32_t kind, flags, slots, nsrc, ndst, ptr_off; };
 
 __device__ __forceinline__ uint32_t uniform32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
@@ -370,19 +370,22 @@ template <bool STAGED>
 __device__ __forceinline__ ColRow column_row(const DevOp* __restrict__ ops, const u4* table, uint32_t j) {
     ColRow r;
     if (STAGED) {
-        const u4 q0 = table[j * 4u], q1 = table[j * 4u + 1u], q3 = table[j * 4u + 3u];
+        const u4 q0 = table[j * 4u], q1 = table[j * 4u + 1u], q2 = table[j * 4u + 2u], q3 = table[j * 4u + 3u];
         r.p0 = reinterpret_cast<char*>((uint64_t)uniform32(q0.x) | ((uint64_t)uniform32(q0.y) << 32));
         r.p1 = reinterpret_cast<char*>((uint64_t)uniform32(q0.z) | ((uint64_t)uniform32(q0.w) << 32));
         r.bytes = (uint64_t)uniform32(q1.x) | ((uint64_t)uniform32(q1.y) << 32);
         r.kind = uniform32(q1.z); r.flags = uniform32(q1.w); r.slots = uniform32(q3.y);
+        r.nsrc = uniform32(q2.z); r.ndst = uniform32(q2.w); r.ptr_off = uniform32(q3.x);
     } else {
         r.p0 = ops[j].p0; r.p1 = ops[j].p1; r.bytes = ops[j].bytes;
         r.kind = ops[j].kind; r.flags = ops[j].flags; r.slots = ops[j].slots;
+        r.nsrc = ops[j].nsrc; r.ndst = ops[j].ndst; r.ptr_off = ops[j].ptr_off;
     }
     return r;
 }
 static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offsetof(DevOp, kind) == 24 &&
-              offsetof(DevOp, flags) == 28 && offsetof(DevOp, slots) == 52, "column_row reads DevOp by position");
+              offsetof(DevOp, flags) == 28 && offsetof(DevOp, nsrc) == 40 && offsetof(DevOp, ndst) == 44 &&
+              offsetof(DevOp, ptr_off) == 48 && offsetof(DevOp, slots) == 52, "column_row reads DevOp by position");
 
 // Rows that share no (rank, chunk) cell never depend on each other, whatever round they sit in.  The host
 // therefore splits the rows into connected components (for all four algorithms: one per chunk index) and a
@@ -396,7 +399,7 @@ static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offset
 // the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.
 template <int DT, int BLOCK, bool FWD, bool LAT, int POL>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
-                                                        const ColumnComp* __restrict__ comps, ColumnLaunch L) {
+                                                        const ColumnComp* __restrict__ comps, char* const* __restrict__ ptrs, ColumnLaunch L) {
     typedef typename Elem<DT>::T T;
     // Vectors per lane and row: two when values are forwarded in the bandwidth regime (the loads that remain are
     // few and far between, and two in flight per lane pay: +2 to +9 %), one otherwise (every row loads and
@@ -443,7 +446,31 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                 const uint64_t bytes = row.bytes;
                 char* const p0 = row.p0;
                 char* const p1 = row.p1;
-                if (flags & DEVOP_VEC) {
+                if (kind == SAR_OP_MREDUCE) {
+                    // Multi-source row (a pre-work collective lowered into the same launch; the host only does that
+                    // when all its pointers are 16-byte aligned and the row is a whole number of vectors long):
+                    // acc = srcs[0]; acc = srcs[k] + acc, the owner's own data last; the result goes to every dst
+                    // and, flagged PUT, into a slot for the exchange that follows.
+                    char* const* const srcs = ptrs + row.ptr_off;
+                    char* const* const dsts = srcs + row.nsrc;
+                    constexpr uint64_t vstep = (uint64_t)BLOCK * 16u;
+#pragma unroll
+                    for (uint32_t v = 0; v < V; ++v) {
+                        const uint64_t o = voff + v * vstep;
+                        if (o + 16u <= bytes) {
+                            f4 acc = ld16<LNT>(srcs[0] + o);
+                            for (uint32_t k0 = 1; k0 < row.nsrc; k0 += 8u) {
+                                f4 t[8];
+#pragma unroll
+                                for (uint32_t q = 0; q < 8u; ++q) if (k0 + q < row.nsrc) t[q] = ld16<LNT>(srcs[k0 + q] + o);
+#pragma unroll
+                                for (uint32_t q = 0; q < 8u; ++q) if (k0 + q < row.nsrc) acc = add16<DT>(t[q], acc);
+                            }
+                            for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(dsts[d] + o, acc);
+                            if (FWD && (flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = acc;
+                        }
+                    }
+                } else if (flags & DEVOP_VEC) {
                     if (voff + 16u <= bytes) {
                         const uint32_t slots = FWD ? row.slots : 0u;
                         const bool get0 = FWD && (flags & DEVOP_GET0), get1 = FWD && (flags & DEVOP_GET1);
@@ -513,9 +540,9 @@ int column_latency_block() { return 256; }
 template <int DT, bool FWD, int POL>
 static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hipStream_t st, const ColumnLaunch& L) {
     switch (block) {
-        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L); break;
-        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L); break;
-        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L); break;
+        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -524,8 +551,8 @@ static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hi
 template <int DT, int POL>
 static hipError_t launch_column_policy(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
     if (L.table_rows) {
-        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L);
-        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L);
+        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
+        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
         return hipGetLastError();
     }
     return fwd ? launch_column_block<DT, true, POL>(block, grid, lds, st, L) : launch_column_block<DT, false, POL>(block, grid, lds, st, L);

@@ -257,6 +257,34 @@ def test_latency_plan_on_many_columns(gpu_ctx, sarlib, oracle, alg):
             assert_bits_equal(got[r], want[r], "%s tuning %r rank %d" % (alg, t, r))
 
 
+@pytest.mark.parametrize("alg,n,table", [("stragglar", 8, "stragglar_n8_cu.txt"), ("stragglar", 6, "synth_nonpow2_n6.txt"),
+                                         ("stragglar", 16, "synth_pow2_n16.txt"), ("direct", 8, None), ("stragglar", 4, "stragglar_n4_cu.txt")])
+def test_prework_in_the_same_launch(gpu_ctx, sarlib, oracle, alg, n, table):
+    """With no delay the pre-work collective and the schedule run as one launch of the column kernel (the
+    pre-work's result is handed to the exchange in a value slot); the buffers must equal the checker's, and those
+    of the pre-work as launches of its own."""
+    text = read_golden(table) if table else None
+    parts = (n - 1) if alg == "stragglar" else 1
+    for dtype, chunk_elems in (("f32", 4096 + 512), ("bf16", 8 * 1030), ("f16", 8 * 52000), ("f32", 4 * 700 + 2)):
+        elems = parts * chunk_elems + (3 if parts > 1 else 0)
+        inputs = make_inputs(n, elems, dtype, seed=44, kind="normal", scale=1.0)
+        want = run_oracle(oracle, alg, inputs, dtype, text, delay=0.0)
+        es = 4 if dtype == "f32" else 2
+        for t in (dict(), dict(col_fuse_prework=0), dict(col_forward=0), dict(col_latency_plan=0), dict(col_latency_plan=2, col_wgs=1),
+                  dict(col_split=0), dict(col_block=512, col_latency_plan=0, cache_policy=0), dict(executor=0)):
+            got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=0.0, tuning=dict(dict(executor=1), **t))
+            st = gpu_ctx.stats()
+            # (direct's pre-work cuts the buffer into n-1 chunks, direct itself moves it whole: never merged)
+            fusable = alg == "stragglar" and t.get("executor", 1) == 1 and t.get("col_fuse_prework", 1) == 1 and ((elems // parts) * es) % 16 == 0
+            assert st.fused_prework == (1 if fusable else 0), (t, dtype, chunk_elems)
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "%s n=%d %s chunk %d tuning %r rank %d" % (alg, n, dtype, chunk_elems, t, r))
+        # a delay keeps the pre-work a launch of its own (it overlaps the straggler's absence)
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=0.05, tuning=dict(executor=1))
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s n=%d %s delayed rank %d" % (alg, n, dtype, r))
+
+
 def test_graph_replays_match_eager(gpu_ctx, sarlib, oracle):
     """The captured graph holds kernel nodes only; every replay, with eager work and synchronisation
     between replays, must equal the eager result."""

@@ -93,6 +93,12 @@ def test_prework_and_misaligned_buffers(sarlib):
     S = sarlib.pad_bytes(16 * MIB, 8)
     st = plan(sarlib, "stragglar", 8, S, delay=True)
     assert st.prework_bytes == 8 * S and st.launches == 2     # one multi-source launch, then the column kernel
+    assert st.fused_prework == 1                              # ... or both as one launch when nobody is late
+    assert plan(sarlib, "stragglar", 8, S, delay=True, col_fuse_prework=0).fused_prework == 0
+    assert plan(sarlib, "stragglar", 8, S, delay=True, executor=0).fused_prework == 0
+    assert plan(sarlib, "stragglar", 8, S).fused_prework == 0
+    # direct's pre-work cuts the buffer into n-1 chunks, direct itself moves it whole: not merged
+    assert plan(sarlib, "direct", 8, S, delay=True).fused_prework == 0
     # chunk of 4k+2 elements: rows keep their alignment only where the chunk offset happens to allow it
     odd = plan(sarlib, "stragglar", 8, 7 * 4 * 1026, col_latency_plan=0)
     assert 0 <= odd.forwarded_bytes < 42 * 4 * 1026
