@@ -231,9 +231,10 @@ int sar_get_tuning(sar_ctx* ctx, sar_tuning_t* out);
 int sar_set_tuning(sar_ctx* ctx, const sar_tuning_t* in);   /* takes effect at the next sar_prepare */
 
 /* Lower `main` (and the optional pre-work run before it in delay mode) onto
- * the allocated ranks: per-round op tables in device memory, launch shapes,
- * and with use_graph != 0 a captured hipGraph of the main rounds.  Replaces
- * the unrolled bodies of the *_allreduce_helper functions. */
+ * the allocated ranks: row tables in device memory for the executor the
+ * tuning selects (see sar_tuning_t), launch shapes, and with use_graph != 0 a
+ * captured hipGraph of the main schedule.  Replaces the unrolled bodies of
+ * the *_allreduce_helper functions. */
 int sar_prepare(sar_ctx* ctx, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph);
 
 /* One timed execution = one call of stragglar_allreduce / ring_allreduce /
@@ -257,13 +258,16 @@ int sar_launch_bytes(sar_ctx* ctx, uint64_t* bytes, int cap, int* count);
  * allreduce_8GPU.cu:47-58, uses ms * clockRate_kHz of the shader clock). */
 int sar_sleep_ticks(sar_ctx* ctx, float delay_ms, int64_t* ticks);
 
+/* What sar_prepare planned (launches, executor, column width, components, value slots, forwarded bytes). */
 int sar_stats(sar_ctx* ctx, sar_stats_t* out);
-/* What sar_prepare would decide for `n` rank buffers of `bytes_per_rank` bytes, worked out on the host alone: no
-   device, no context, nothing is allocated (launches, executor, column width, components, value slots, forwarded
-   bytes).  `tuning` NULL = the defaults; `compute_units` 0 = 256 (MI355X).  No counterpart in the reference, whose
-   executors are fixed code (allreduce_8GPU.cu:555-874); meant for tools and tests that inspect a plan. */
-/* the tuning a new context starts with (no device needed) */
+
+/* The tuning a new context starts with (no device needed). */
 int sar_default_tuning(sar_tuning_t* out);
+
+/* What sar_prepare would decide for `n` rank buffers of `bytes_per_rank` bytes, worked out on the host alone:
+ * no device, no context, nothing is allocated.  `tuning` NULL = the defaults; `compute_units` 0 = 256 (MI355X).
+ * No counterpart in the reference, whose executors are fixed code (allreduce_8GPU.cu:555-874); meant for tools
+ * and tests that inspect a plan. */
 int sar_plan(const sar_schedule* prework, const sar_schedule* main_schedule, int n, uint64_t bytes_per_rank, int dtype,
              const sar_tuning_t* tuning, int compute_units, sar_stats_t* out);
 
