@@ -47,7 +47,7 @@ struct ColumnDevice {
     bool ready = false;
     uint32_t* d_group_begin = nullptr;
     sar::ColumnComp* d_comps = nullptr;
-    uint32_t first_op = 0, ncomp = 0, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0;
+    uint32_t first_op = 0, ncomp = 0, ncols = 0, run = 1, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0;
 };
 
 struct sar_ctx {
@@ -316,6 +316,7 @@ struct ColumnPlan {
     bool staged = false;             // latency plan: a workgroup copies the rows of its component into LDS first
     uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
     bool unsupported = false;        // the rows cannot all run in the column kernel
+    bool component_major = false;    // dispatch order of the items: all columns of a component, then the next component
 };
 
 // `scheds`: the schedules to run back to back in the one launch (the main schedule, or pre-work + main); they share
@@ -590,6 +591,29 @@ int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, st
     // 4-10 % there).  Streaming stores never paid in this kernel (-3 to -25 %).
     plan.policy = c->tune.cache_policy == 0 ? 0u : c->tune.cache_policy == 1 ? 2u : c->tune.cache_policy == 3 ? 1u : (all_found ? 1u : 0u);
 
+    // Dispatch order of the items.  All columns of one component before the next component keeps the resident
+    // workgroups on few (rank, chunk) streams at a time (+3 to +5 % for the StragglAR tables, +2 % for ring at 64 MiB
+    // per rank and more).  It only matters, and only pays, when the items outnumber the resident workgroups
+    // severalfold and every row is vector-aligned; and it does not pay where a component reduces several pairs of
+    // ranks in the same round (halving-doubling: -4 to -15 %).  Otherwise the items of one column, all components,
+    // are dispatched together.
+    {
+        uint32_t most = 0;
+        bool aligned = true;
+        for (size_t g = 0; g + 1 < plan.group_begin.size(); ++g) {
+            uint32_t reducing = 0;
+            for (uint32_t i = plan.group_begin[g]; i < plan.group_begin[g + 1]; ++i) {
+                reducing += cr[i].d.kind != SAR_OP_COPY;
+                aligned &= (cr[i].d.flags & sar::DEVOP_VEC) != 0;
+            }
+            most = std::max(most, reducing);
+        }
+        const uint64_t cbytes = sar::column_bytes(plan.block, plan.nslots != 0 && !plan.staged);
+        const uint64_t items = (plan.widest_row + cbytes - 1) / cbytes * plan.comps.size();
+        const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (2048u / (uint32_t)plan.block);
+        plan.component_major = most <= 1 && aligned && !plan.staged && items >= 2 * resident;
+    }
+
     plan.lane_local = true;
     for (const auto& r : cr) {
         if (!(r.d.flags & sar::DEVOP_VEC) || (r.d.bytes & 15u)) plan.lane_local = false;
@@ -640,6 +664,7 @@ int launch_column_plan(sar_ctx* c, const ColumnDevice& d) {
     L.ncomp = d.ncomp; L.nitems = d.items;
     L.table_rows = d.table_rows; L.table_groups = d.table_groups;
     L.lane_local = d.lane_local; L.policy = d.policy;
+    L.ncols = d.ncols; L.run = d.run;
     SAR_HIP(sar::launch_column(c->dtype, (int)d.block, d.grid, d.slots, c->stream, L));
     return SAR_OK;
 }
@@ -660,7 +685,9 @@ int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, Colu
     d.table_rows = cp.staged ? cp.max_comp_rows : 0u;
     d.table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
     d.policy = cp.policy;
-    d.first_op = first_op; d.ncomp = (uint32_t)cp.comps.size(); d.items = (uint32_t)items;
+    d.first_op = first_op; d.ncomp = (uint32_t)cp.comps.size(); d.ncols = (uint32_t)ncols;
+    d.run = cp.component_major ? (uint32_t)ncols : 1u;        // d.run divides ncols either way: no padding items
+    d.items = (uint32_t)items;
     const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
     d.grid = (uint32_t)std::min<uint64_t>(items, resident);
     d.ready = true;

@@ -420,7 +420,11 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
     f4* const mine = reinterpret_cast<f4*>(lds_raw) + table_vecs + group_vecs + threadIdx.x;
     bool first_item = true;
     for (uint32_t item = blockIdx.x; item < L.nitems; item += gridDim.x) {
-        const uint32_t comp = item % L.ncomp, col = item / L.ncomp;
+        // items in dispatch order: `run` neighbouring columns of one component, then the same columns of the next
+        // component, ...; then the next `run` columns
+        const uint32_t per_block = L.run * L.ncomp, blk = item / per_block, within = item - blk * per_block;
+        const uint32_t comp = within / L.run, col = blk * L.run + within % L.run;
+        if (col >= L.ncols) continue;
         const ColumnComp C = comps[comp];
         if (LAT) {
             // Few workgroups, nobody to warm the scalar cache: a row read through scalar loads costs a trip to

@@ -55,7 +55,8 @@ struct ColumnLaunch {
     const uint32_t* group_begin; // rows of group g are ops[group_begin[g] .. group_begin[g+1])
     const ColumnComp* comps;
     char* const* ptrs;           // pointer lists of MREDUCE rows (srcs, then dsts, from the row's ptr_off)
-    uint32_t ncomp, nitems;      // nitems = ncomp * number of columns; item i is component i % ncomp of column i / ncomp
+    uint32_t ncomp, ncols, run;  // items in dispatch order: `run` neighbouring columns of component 0, the same columns of
+    uint32_t nitems;             // component 1, ...; then the next `run` columns.  nitems = ceil(ncols / run) * run * ncomp
     uint32_t table_rows;         // 0, or the most rows of a component: latency plan, the workgroup copies the rows and
     uint32_t table_groups;       // group boundaries (at most table_groups) of its component into LDS first (block =
                                  // column_latency_block())
