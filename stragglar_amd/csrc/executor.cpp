@@ -419,6 +419,27 @@ int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, st
         cr.swap(sorted);
     }
 
+    // Chunks that do not start on a 16-byte boundary (a buffer cut into a number of parts that its size was not
+    // padded for).  When all rows of a component start the same distance h in front of a boundary, on both sides,
+    // they are moved up to it and run as vectors; the h bytes in front are done element by element in the first
+    // column.  All rows of a component must move together: a column has to mean the same offsets in each of them.
+    for (const auto& cc : plan.comps) {
+        const uint32_t phase = (uint32_t)((uintptr_t)cr[cc.row_first].d.p0 & 15u), h = 16u - phase;
+        bool same = phase != 0 && phase % (uint32_t)es == 0;
+        for (uint32_t i = cc.row_first; i < cc.row_end && same; ++i) {
+            const sar::DevOp& d = cr[i].d;
+            same = d.kind != SAR_OP_MREDUCE && ((uintptr_t)d.p0 & 15u) == phase && ((uintptr_t)d.p1 & 15u) == phase && d.bytes > h;
+        }
+        if (!same) continue;
+        for (uint32_t i = cc.row_first; i < cc.row_end; ++i) {
+            sar::DevOp& d = cr[i].d;
+            d.p0 += h; d.p1 += h; d.bytes -= h;
+            d.flags |= sar::DEVOP_VEC | (h << sar::DEVOP_HEAD_SHIFT);
+        }
+    }
+    plan.widest_row = 0;
+    for (const auto& r : cr) plan.widest_row = std::max(plan.widest_row, r.d.bytes);
+
     // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
     plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512, false) >= 2048 ? 512 : 256);
 
@@ -616,7 +637,7 @@ int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, st
 
     plan.lane_local = true;
     for (const auto& r : cr) {
-        if (!(r.d.flags & sar::DEVOP_VEC) || (r.d.bytes & 15u)) plan.lane_local = false;
+        if (!(r.d.flags & sar::DEVOP_VEC) || (r.d.bytes & 15u) || (r.d.flags >> sar::DEVOP_HEAD_SHIFT & 15u)) plan.lane_local = false;
         rows.push_back(r.d);
     }
     return SAR_OK;

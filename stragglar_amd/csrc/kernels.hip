@@ -519,6 +519,16 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                         *reinterpret_cast<T*>(p0 + o) = s;
                         if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
                     }
+                    // the < 16 bytes in front of p0 and p1 of a row that was moved up to a 16-byte boundary, in
+                    // the first column (through memory as well)
+                    const uint32_t head = (flags >> DEVOP_HEAD_SHIFT & 15u) / (uint32_t)sizeof(T);
+                    if (head && off == 0 && threadIdx.x < head) {
+                        const int64_t o = ((int64_t)threadIdx.x - (int64_t)head) * (int64_t)sizeof(T);
+                        T s = *reinterpret_cast<const T*>(p1 + o);
+                        if (kind != SAR_OP_COPY) s = add1<DT>(*reinterpret_cast<const T*>(p0 + o), s);
+                        *reinterpret_cast<T*>(p0 + o) = s;
+                        if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
+                    }
                 } else if (off < bytes) {                               // row not 16-byte aligned: element by element
                     const uint64_t rem = bytes - off;
                     const uint32_t len = rem < col_bytes ? (uint32_t)rem : (uint32_t)col_bytes;

@@ -15,7 +15,9 @@ enum : uint32_t {
     DEVOP_VEC = 8u,    // every pointer of the row is 16-byte aligned
     DEVOP_GET0 = 16u,  // column executor: p0's current value is in value slot (slots & 0xff)
     DEVOP_GET1 = 32u,  // column executor: p1's current value is in value slot (slots >> 8 & 0xff)
-    DEVOP_PUT = 64u    // column executor: keep the row's result in value slot (slots >> 16 & 0xff)
+    DEVOP_PUT = 64u,   // column executor: keep the row's result in value slot (slots >> 16 & 0xff)
+    DEVOP_HEAD_SHIFT = 8u  // column executor: flags >> 8 & 15 = bytes of the row that lie before p0 and p1 (both moved
+                           // up to the next 16-byte boundary; `bytes` counts from there)
 };
 
 // One lowered row of a round, read by the kernel through scalar loads.

@@ -117,3 +117,18 @@ def test_plan_argument_checks(sarlib):
         sarlib.plan(main, 8, 1 << 20, col_block=333)
     with pytest.raises(KeyError):
         sarlib.plan(main, 8, 1 << 20, no_such_knob=1)
+
+
+def test_chunks_off_the_vector_boundary_are_still_forwarded(sarlib):
+    """A buffer padded for n-1 chunks and cut into n (ring on the n=6 sizes of pad_buffers.py:31-48): the chunks
+    start 0, 4, 8, 12, 0, 4 bytes past a 16-byte boundary.  The rows of one chunk index move up to the boundary
+    together, so their re-reads are found in the value slots as for aligned chunks, less the bytes in front of
+    the first and behind the last whole vector."""
+    S = sarlib.pad_bytes(64 * MIB, 6)
+    chunk = (S // 4 // 6) * 4
+    assert chunk % 16 == 4
+    ring = plan(sarlib, "ring", 6, S)
+    assert ring.executor == 1 and ring.col_components == 6 and ring.col_slots == 1
+    heads = [(16 - (c * chunk) % 16) % 16 for c in range(6)]
+    tails = [(chunk - h) % 16 for h in heads]
+    assert ring.forwarded_bytes == 9 * (6 * chunk - sum(heads) - sum(tails))     # 4 of 5 reduce-scatter reads + 5 all-gather copies per chunk
