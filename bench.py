@@ -173,10 +173,12 @@ def main():
                 "kernel": "sar::column_kernel<f32, %d, %s>" % (st.col_block, "forwarding" if st.col_slots else "no forwarding") if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
                 "launches": len(launch_bytes),
                 "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
-    if st.forwarded_bytes:
-        roofline["note"] = ("frac can pass 1: %.1f %% of the algorithmic bytes are re-reads of values the same lane wrote, served from LDS; "
+    kept_on_chip = st.forwarded_bytes + st.elided_store_bytes
+    if kept_on_chip:
+        roofline["note"] = ("frac can pass 1: %.1f %% of the algorithmic bytes are re-reads of values the same lane wrote, served from LDS%s; "
                             "the memory side (traffic) ran at %.0f GB/s" % (100.0 * st.forwarded_bytes / st.algorithmic_bytes,
-                                                                          (mean_launch_bytes - st.forwarded_bytes / len(launch_bytes)) / mean_launch_ms / 1e6))
+                                                                          ", and %.1f %% are stores of partial sums that are overwritten unread and left out" % (100.0 * st.elided_store_bytes / st.algorithmic_bytes) if st.elided_store_bytes else "",
+                                                                          (mean_launch_bytes - kept_on_chip / len(launch_bytes)) / mean_launch_ms / 1e6))
     # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
     rec = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -188,9 +190,11 @@ def main():
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
         # part of the algorithmic bytes that never leaves the compute unit: re-reads of values the same lane wrote
-        # in an earlier round, taken from LDS slots (every store still goes to the rank buffers)
+        # in an earlier round, taken from LDS slots
         "forwarded_bytes_per_step": int(st.forwarded_bytes),
-        "memory_side_GBps": round((st.algorithmic_bytes - st.forwarded_bytes) / ms / 1e6, 1),
+        # stores of values that a later row overwrites before anybody loads them (none in the StragglAR tables)
+        "elided_store_bytes_per_step": int(st.elided_store_bytes),
+        "memory_side_GBps": round((st.algorithmic_bytes - st.forwarded_bytes - st.elided_store_bytes) / ms / 1e6, 1),
         "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),
         "wall_ms_per_step_back_to_back": round(back_to_back_ms, 4),
         "ranks_identical_after_run": bool(identical),

@@ -83,6 +83,8 @@ typedef struct sar_stats_t {
                                    /* in LDS instead of loading it again from the rank buffers                    */
     int32_t fused_prework;         /* 1 if sar_run(delay 0) runs pre-work + main schedule as a single launch      */
     int32_t reserved;
+    uint64_t elided_store_bytes;   /* part of algorithmic_bytes that the column executor does not store because a */
+                                   /* later row overwrites it and every reader in between takes it from a slot    */
 } sar_stats_t;
 
 /* run-time tunables of the executors; sar_get_tuning() reports the defaults */
@@ -108,8 +110,8 @@ typedef struct sar_tuning_t {
     int32_t col_block;    /* column executor: threads per workgroup = 16-byte vectors per column     */
                           /*     (256, 512 or 1024; 0 = chosen from the number of columns)           */
     int32_t col_forward;  /* column executor: 1 = a value a lane wrote in an earlier round and needs  */
-                          /*     again is kept in LDS and not loaded again (all stores still happen; */
-                          /*     same bits); 0 = every operand is loaded from its rank buffer        */
+                          /*     again is kept in LDS and not loaded again (same bits);              */
+                          /*     0 = every operand is loaded from its rank buffer                    */
     int32_t col_slots;    /* column executor: most values kept per lane (0 = chosen by the planner)  */
     int32_t col_light_sync; /* column executor: 1 = between rounds the waves of a workgroup only meet   */
                           /*     (no wait for their stores) whenever no lane reads bytes another lane */
@@ -125,6 +127,10 @@ typedef struct sar_tuning_t {
                           /*     schedule as one launch (the pre-work's result for a chunk goes to   */
                           /*     that chunk's exchange in a value slot); with a delay the pre-work   */
                           /*     stays a launch of its own, overlapping the straggler's absence      */
+    int32_t col_elide_stores; /* column executor: 1 = a forwarded value whose stored copy nobody loads  */
+                          /*     before a later row overwrites it (partial sums of ring and halving- */
+                          /*     doubling, the pre-work's result in a same-launch run) is not stored;*/
+                          /*     the buffers after sar_run are the same either way                  */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

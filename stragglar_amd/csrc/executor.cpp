@@ -63,7 +63,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -312,6 +312,7 @@ struct ColumnPlan {
     int block = 512;
     uint32_t nslots = 0;
     uint64_t forwarded_bytes = 0;    // operand bytes taken from value slots instead of memory, per run
+    uint64_t elided_bytes = 0;       // result bytes not stored because they are overwritten unread, per run
     bool lane_local = false;         // every row 16-byte aligned and a whole number of vectors long
     bool staged = false;             // latency plan: a workgroup copies the rows of its component into LDS first
     uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
@@ -333,7 +334,7 @@ int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, st
     };
     struct ColRow { sar::DevOp d; int c0, c1; uint32_t round; std::vector<int> mreads, mwrites; };   // m*: cells of a multi-source row
     std::vector<ColRow> cr;
-    plan.group_begin.clear(); plan.comps.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0; plan.unsupported = false;
+    plan.group_begin.clear(); plan.comps.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0; plan.elided_bytes = 0; plan.unsupported = false;
     uint32_t round_no = 0;
     for (const sar::Schedule* sp : scheds) {
       if (sp->parts != s.parts) { plan.unsupported = true; return SAR_OK; }
@@ -604,6 +605,42 @@ int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, st
         }
     }
     plan.nslots = fwd.nslots; plan.forwarded_bytes = fwd.bytes;
+
+    // Stores nobody needs.  A row's result for a cell is dead when a later row overwrites the cell and every row
+    // that reads it before then (the overwriting row included, if it reads) takes it from a slot: the partial
+    // sums of ring and halving-doubling, the pre-work's result ahead of the exchange in a same-launch run.  Only
+    // the whole vectors are left out; the bytes in front of the first and behind the last one always go through
+    // memory.  What the rank buffers hold after the launch does not change.
+    if (fwd.nslots && c->tune.col_elide_stores) {
+        auto from_slot = [&](uint32_t j, int cell) {            // does row j take the cell's value from a slot?
+            const sar::DevOp& d = cr[j].d;
+            if (d.kind == SAR_OP_MREDUCE || cr[j].c0 == cr[j].c1) return false;
+            if (cell == cr[j].c1) return (fwd.flags[j] & sar::DEVOP_GET1) != 0;
+            return cell == cr[j].c0 && d.kind != SAR_OP_COPY && (fwd.flags[j] & sar::DEVOP_GET0) != 0;
+        };
+        auto dead = [&](uint32_t i, int cell) {
+            if (!(cr[i].d.flags & sar::DEVOP_VEC)) return false;
+            const auto& v = ev[(size_t)cell];
+            for (auto it = std::upper_bound(v.begin(), v.end(), i, [](uint32_t x, const Ev& e) { return x < e.row; }); it != v.end(); ++it) {
+                if (it->reads && !from_slot(it->row, cell)) return false;
+                if (it->writes) return (cr[it->row].d.flags & sar::DEVOP_VEC) && cr[it->row].d.bytes == cr[i].d.bytes;
+            }
+            return false;                                       // never overwritten: part of the result
+        };
+        for (uint32_t i = 0; i < nrows; ++i) {
+            const sar::DevOp& d = cr[i].d;
+            const uint64_t vec_bytes = d.bytes & ~(uint64_t)15u;
+            if (d.kind == SAR_OP_MREDUCE) {
+                bool all = true;
+                for (int cell : cr[i].mwrites) all = all && dead(i, cell);
+                if (all) { fwd.flags[i] |= sar::DEVOP_DEAD0; plan.elided_bytes += vec_bytes * d.ndst; }
+                continue;
+            }
+            if (cr[i].c0 == cr[i].c1) continue;
+            if (dead(i, cr[i].c0)) { fwd.flags[i] |= sar::DEVOP_DEAD0; plan.elided_bytes += vec_bytes; }
+            if (d.kind == SAR_OP_XREDUCE && dead(i, cr[i].c1)) { fwd.flags[i] |= sar::DEVOP_DEAD1; plan.elided_bytes += vec_bytes; }
+        }
+    }
     for (uint32_t i = 0; i < nrows; ++i) { cr[i].d.flags |= fwd.flags[i]; cr[i].d.slots = fwd.slots[i]; }
 
     // Cache policy of the launch (the column kernel takes one for all its rows).  Planned (2): when every re-read is
@@ -670,7 +707,7 @@ bool column_pays(const sar_ctx* c, const ColumnPlan& cp) {
     const double passes = std::ceil(items / resident);
     double est_stream;
     if (cp.nslots) {
-        const double to_memory = std::max(0.0, bytes - (double)cp.forwarded_bytes);
+        const double to_memory = std::max(0.0, bytes - (double)cp.forwarded_bytes - (double)cp.elided_bytes);
         est_stream = to_memory / ((double)cp.forwarded_bytes >= 0.3 * bytes ? 5.0e6 : 6.0e6);             // bytes per us
     } else {
         est_stream = bytes / (item_rows <= 128 ? 7.1e6 : item_rows <= 256 ? 6.4e6 : 5.3e6);
@@ -777,6 +814,7 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     st.col_slots = column ? (int32_t)cp.nslots : 0;
     st.col_components = column ? (int32_t)cp.comps.size() : 0;
     st.forwarded_bytes = column ? cp.forwarded_bytes : 0;
+    st.elided_store_bytes = column ? cp.elided_bytes : 0;
     st.fused_prework = fused ? 1 : 0;
     return st;
 }
@@ -789,7 +827,8 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024) &&
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
-           (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1);
+           (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
+           (t.col_elide_stores == 0 || t.col_elide_stores == 1);
 }
 
 }  // namespace

@@ -470,7 +470,7 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
 #pragma unroll
                                 for (uint32_t q = 0; q < 8u; ++q) if (k0 + q < row.nsrc) acc = add16<DT>(t[q], acc);
                             }
-                            for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(dsts[d] + o, acc);
+                            if (!(FWD && (flags & DEVOP_DEAD0))) for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(dsts[d] + o, acc);
                             if (FWD && (flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = acc;
                         }
                     }
@@ -479,13 +479,14 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                         const uint32_t slots = FWD ? row.slots : 0u;
                         const bool get0 = FWD && (flags & DEVOP_GET0), get1 = FWD && (flags & DEVOP_GET1);
                         constexpr uint64_t vstep = (uint64_t)BLOCK * 16u;
+                        const bool live0 = !(FWD && (flags & DEVOP_DEAD0)), live1 = !(FWD && (flags & DEVOP_DEAD1));
                         if (FWD && kind == SAR_OP_COPY && get1) {
                             // A copy of a held value is a store and nothing else.  It has a path of its own so
                             // that it does not pass the wait for loaded operands below: the memory counter
                             // runs in order, and that wait would also sit out the stores of the rows before.
 #pragma unroll
                             for (uint32_t v = 0; v < V; ++v)
-                                if (voff + v * vstep + 16u <= bytes) st16<SNT>(p0 + voff + v * vstep, mine[((slots >> 8 & 0xffu) * V + v) * BLOCK]);
+                                if (live0 && voff + v * vstep + 16u <= bytes) st16<SNT>(p0 + voff + v * vstep, mine[((slots >> 8 & 0xffu) * V + v) * BLOCK]);
                         } else {
                             f4 a[V], b[V];
 #pragma unroll
@@ -501,8 +502,8 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                                 const uint64_t o = voff + v * vstep;
                                 if (o + 16u <= bytes) {
                                     const f4 s = kind == SAR_OP_COPY ? b[v] : add16<DT>(a[v], b[v]);
-                                    st16<SNT>(p0 + o, s);
-                                    if (kind == SAR_OP_XREDUCE) st16<SNT>(p1 + o, s);
+                                    if (live0) st16<SNT>(p0 + o, s);
+                                    if (kind == SAR_OP_XREDUCE && live1) st16<SNT>(p1 + o, s);
                                     if (FWD && (flags & DEVOP_PUT)) mine[((slots >> 16 & 0xffu) * V + v) * BLOCK] = s;
                                 }
                             }

@@ -16,6 +16,10 @@ enum : uint32_t {
     DEVOP_GET0 = 16u,  // column executor: p0's current value is in value slot (slots & 0xff)
     DEVOP_GET1 = 32u,  // column executor: p1's current value is in value slot (slots >> 8 & 0xff)
     DEVOP_PUT = 64u,   // column executor: keep the row's result in value slot (slots >> 16 & 0xff)
+    DEVOP_DEAD0 = 128u,    // column executor: the whole vectors stored to p0 (MREDUCE: to every destination) are
+                           // overwritten before anybody loads them (every reader in between takes the value from
+                           // a slot): not stored
+    DEVOP_DEAD1 = 4096u,   // the same for p1 (XREDUCE)
     DEVOP_HEAD_SHIFT = 8u  // column executor: flags >> 8 & 15 = bytes of the row that lie before p0 and p1 (both moved
                            // up to the next 16-byte boundary; `bytes` counts from there)
 };

@@ -209,7 +209,7 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
         elems = parts * chunk_elems + (2 if parts > 1 else 0)
         inputs = make_inputs(n, elems, dtype, seed=21, kind="normal", scale=1.0)
         want = run_oracle(oracle, alg, inputs, dtype, text, delay=-1.0)
-        seen = set()
+        seen, elided = set(), set()
         for t in (dict(col_forward=0), dict(col_forward=1), dict(col_forward=1, col_slots=1), dict(col_forward=1, col_slots=2),
                   dict(col_forward=1, col_slots=3, col_block=512), dict(col_forward=1, col_slots=5, col_light_sync=0),
                   dict(col_forward=1, col_slots=16, col_block=256), dict(col_forward=1, col_slots=255, col_block=1024),
@@ -217,11 +217,15 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
                   dict(col_forward=1, cache_policy=3), dict(col_forward=0, cache_policy=3),
                   dict(col_forward=1, col_latency_plan=1), dict(col_forward=1, col_latency_plan=2, col_slots=2),
                   dict(col_forward=0, col_latency_plan=2, cache_policy=1),
-                  dict(col_forward=1, col_split=0), dict(col_forward=0, col_split=0), dict(col_forward=1, col_split=0, col_latency_plan=2)):
+                  dict(col_forward=1, col_split=0), dict(col_forward=0, col_split=0), dict(col_forward=1, col_split=0, col_latency_plan=2),
+                  dict(col_forward=1, col_elide_stores=0), dict(col_forward=1, col_elide_stores=0, col_slots=2, col_latency_plan=2)):
             # these buffers have few columns: unless a case asks for it, keep the plan for few work items out of the way
             got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(dict(col_latency_plan=0), **dict(t, executor=1)))
             st = gpu_ctx.stats()
             assert st.executor == 1
+            assert st.elided_store_bytes <= st.forwarded_bytes
+            if not t.get("col_elide_stores", 1):
+                assert st.elided_store_bytes == 0
             if not t["col_forward"]:
                 assert st.forwarded_bytes == 0 and st.col_slots == 0
             else:
@@ -229,11 +233,16 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
                 assert st.forwarded_bytes <= st.algorithmic_bytes
                 assert st.forwarded_bytes == 0 or st.col_slots > 0
             seen.add(st.forwarded_bytes)
+            elided.add(st.elided_store_bytes)
             for r in range(n):
                 assert_bits_equal(got[r], want[r], "%s n=%d %s chunk %d tuning %r rank %d" % (alg, n, dtype, chunk_elems, t, r))
         es = 4 if dtype == "f32" else 2
         if (chunk_elems * es) % 16 == 0:
             assert max(seen) > 0, "aligned rows: some operand must have been forwarded"
+        if (chunk_elems * es) % 16 == 0:
+            # partial sums that are overwritten unread are not stored: all but the last reducing step of every chunk
+            # of ring and halving-doubling; the other tables have no such store
+            assert max(elided) == (n * (n - 2) * chunk_elems * es if alg in ("ring", "rhd") else 0)
         if alg == "stragglar" and (chunk_elems * es) % 16 == 0:
             # every re-read found in a slot: the n-1 ranks' (n-2) copies each of one chunk
             assert max(seen) == (n - 1) * (n - 2) * chunk_elems * es

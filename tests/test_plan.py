@@ -57,6 +57,11 @@ def test_comparators_n8_plan(sarlib):
     # per chunk: 6 of the 7 reduce-scatter steps read the partial sum of the step before, and all 7 all-gather
     # steps copy the held result
     assert ring.forwarded_bytes == 8 * 13 * Cn
+    # and the partial sums of the first 6 reduce-scatter steps are overwritten by the all-gather without ever
+    # being loaded: not stored
+    assert ring.elided_store_bytes == 8 * 6 * Cn
+    assert plan(sarlib, "ring", 8, S, col_elide_stores=0).elided_store_bytes == 0
+    assert plan(sarlib, "ring", 8, S, col_forward=0).elided_store_bytes == 0
     rhd = plan(sarlib, "rhd", 8, S)
     assert rhd.algorithmic_bytes == 35 * S and rhd.rounds == 6
     assert rhd.col_components == 8 and rhd.col_slots == 4     # a butterfly over 8 ranks: 4, 2, 1 partial sums alive
