@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "column_plan.hpp"
 #include "kernels.hpp"
 #include "sar.h"
 #include "schedule.hpp"
@@ -293,391 +294,20 @@ int lower(sar_ctx* c, const sar::Schedule& s, std::vector<sar::DevOp>& rows, std
     return SAR_OK;
 }
 
-// Column plan: every row of the main schedule, cut into single-chunk rows (all rows then share one
-// within-chunk offset space), in round order, plus the index of each round's first row.
-//
-// Value forwarding.  A lane of the column kernel meets the same (rank, chunk) cells again and again: what
-// round r writes, later rounds read back.  The kernel can keep up to `nslots` such values per lane in LDS
-// (write-through: every value is stored to its rank buffer as well), and which read finds its operand
-// there is decided here, on the host, by running the slot bookkeeping over the rows once: a slot stands
-// for one value and the set of cells that currently equal it (a COPY from a held value adds its
-// destination to the set at no cost; a write to a cell takes it out of its old set).  When all slots
-// are busy the value whose next use is furthest away gives way, which is known exactly because the
-// whole schedule is.  Rows get DEVOP_GET0 / GET1 / PUT and their slot numbers.
-struct ColumnPlan {
-    std::vector<uint32_t> group_begin;       // first row of every group (rows of one component and one round), plus the end
-    std::vector<sar::ColumnComp> comps;
-    uint32_t max_comp_rows = 0, max_comp_groups = 0;
-    uint64_t widest_row = 0;
-    int block = 512;
-    uint32_t nslots = 0;
-    uint64_t forwarded_bytes = 0;    // operand bytes taken from value slots instead of memory, per run
-    uint64_t elided_bytes = 0;       // result bytes not stored because they are overwritten unread, per run
-    bool lane_local = false;         // every row 16-byte aligned and a whole number of vectors long
-    bool staged = false;             // latency plan: a workgroup copies the rows of its component into LDS first
-    uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
-    bool unsupported = false;        // the rows cannot all run in the column kernel
-    bool component_major = false;    // dispatch order of the items: all columns of a component, then the next component
-};
+using sar::ColumnPlan;
 
-// `scheds`: the schedules to run back to back in the one launch (the main schedule, or pre-work + main); they share
-// `parts`.  Multi-source rows (pre-work) are only taken when every pointer is 16-byte aligned and the row is a whole
-// number of vectors long; otherwise plan.unsupported is set and the caller keeps the pre-work as launches of its own.
-int lower_column(sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, std::vector<sar::DevOp>& rows, std::vector<char*>& ptrs, ColumnPlan& plan) {
-    const sar::Schedule& s = *scheds.back();
-    const int es = elem_size_of(c->dtype);
-    const uint64_t elems = c->elems();
-    const uint64_t chunk_bytes = (elems / (uint64_t)s.parts) * es;
-    const int cells_per_rank = s.parts + 1;
-    auto cell_of = [&](int rank, uint64_t byte_off) {
-        return rank * cells_per_rank + (int)(chunk_bytes ? std::min<uint64_t>(byte_off / chunk_bytes, (uint64_t)s.parts) : 0);
-    };
-    struct ColRow { sar::DevOp d; int c0, c1; uint32_t round; std::vector<int> mreads, mwrites; };   // m*: cells of a multi-source row
-    std::vector<ColRow> cr;
-    plan.group_begin.clear(); plan.comps.clear(); plan.widest_row = 0; plan.nslots = 0; plan.forwarded_bytes = 0; plan.elided_bytes = 0; plan.unsupported = false;
-    uint32_t round_no = 0;
-    for (const sar::Schedule* sp : scheds) {
-      if (sp->parts != s.parts) { plan.unsupported = true; return SAR_OK; }
-      for (size_t ri = 0; ri < sp->rounds.size(); ++ri, ++round_no) {
-        for (const sar::Op& op : sp->rounds[ri]) {
-            sar::Range rg = sar::lower_range(*sp, op, elems);
-            const uint64_t row_bytes = rg.len * es;
-            if (row_bytes == 0) continue;
-            const uint64_t row_doff = rg.dst_off * es, row_soff = rg.src_off * es;
-            if (row_doff + row_bytes > c->bytes_per_rank || row_soff + row_bytes > c->bytes_per_rank) return set_error(SAR_ESCHED, "row leaves the rank buffer");
-            for (int j = 0; j < op.nchunks; ++j) {
-                const uint64_t base = (uint64_t)j * chunk_bytes;
-                ColRow r{};
-                r.d.kind = (uint32_t)op.kind;
-                r.d.bytes = (j == op.nchunks - 1) ? row_bytes - base : chunk_bytes;     // a to_end row ends with a longer chunk
-                r.round = round_no;
-                if (op.kind == SAR_OP_MREDUCE) {
-                    // ring order over the group: x_{r+1}, x_{r+2}, ..., x_{r-1}, x_r (the owner last), as one launch per round has it
-                    const uint64_t off = row_doff + base;
-                    r.d.ptr_off = (uint32_t)ptrs.size(); r.d.nsrc = (uint32_t)op.group;
-                    for (int q = 1; q <= op.group; ++q) { const int rank = (op.dst_rank + q) % op.group; ptrs.push_back(c->rank_base(rank) + off); r.mreads.push_back(cell_of(rank, off)); }
-                    if (op.bcast) { r.d.ndst = (uint32_t)op.group; for (int q = 0; q < op.group; ++q) { ptrs.push_back(c->rank_base(q) + off); r.mwrites.push_back(cell_of(q, off)); } }
-                    else { r.d.ndst = 1; ptrs.push_back(c->rank_base(op.dst_rank) + off); r.mwrites.push_back(cell_of(op.dst_rank, off)); }
-                    bool aligned = (r.d.bytes & 15u) == 0;
-                    for (size_t k = r.d.ptr_off; k < ptrs.size(); ++k) aligned &= ((uintptr_t)ptrs[k] & 15u) == 0;
-                    if (!aligned) { plan.unsupported = true; return SAR_OK; }
-                    r.d.flags = sar::DEVOP_VEC;
-                    r.d.p0 = ptrs[r.d.ptr_off + r.d.nsrc]; r.d.p1 = ptrs[r.d.ptr_off];
-                    r.c0 = r.mwrites[0]; r.c1 = r.mreads[0];
-                } else {
-                    r.d.p0 = c->rank_base(op.dst_rank) + row_doff + base;
-                    r.d.p1 = c->rank_base(op.src_rank) + row_soff + base;
-                    r.d.flags = ((((uintptr_t)r.d.p0 | (uintptr_t)r.d.p1) & 15u) == 0) ? sar::DEVOP_VEC : 0u;
-                    r.c0 = cell_of(op.dst_rank, row_doff + base);
-                    r.c1 = cell_of(op.src_rank, row_soff + base);
-                }
-                plan.widest_row = std::max(plan.widest_row, r.d.bytes);
-                cr.push_back(r);
-            }
-        }
-      }
-    }
-    if (cr.size() > 0x7ffffff0ull) return set_error(SAR_EINVAL, "schedule has too many rows");
-    const uint32_t nrows = (uint32_t)cr.size();
-    const uint32_t never = 0xffffffffu;
-    const int ncells = c->n * cells_per_rank;
+sar::ColumnEnv column_env(const sar_ctx* c) {
+    sar::ColumnEnv env;
+    env.tune = c->tune; env.n = c->n; env.elem_size = elem_size_of(c->dtype); env.elems = c->elems();
+    env.bytes_per_rank = c->bytes_per_rank; env.compute_units = c->cu_count;
+    for (int r = 0; r < c->n; ++r) env.rank_base.push_back(c->rank_base(r));
+    return env;
+}
 
-    // Components: rows that (transitively) share a cell.  Rows of different components touch disjoint bytes in
-    // every column, so no order is needed between them; within a component the round order is kept.  For the
-    // four algorithms every row moves a chunk to the same chunk index, and the components are the chunk indices.
-    {
-        std::vector<int> parent((size_t)ncells);
-        for (int i = 0; i < ncells; ++i) parent[(size_t)i] = i;
-        auto find = [&](int x) { while (parent[(size_t)x] != x) { parent[(size_t)x] = parent[(size_t)parent[(size_t)x]]; x = parent[(size_t)x]; } return x; };
-        auto unite = [&](int x, int y) { const int a = find(x), b2 = find(y); if (a != b2) parent[(size_t)b2] = a; };
-        if (c->tune.col_split) for (const auto& r : cr) {
-            unite(r.c0, r.c1);
-            for (int cell : r.mreads) unite(r.c0, cell);
-            for (int cell : r.mwrites) unite(r.c0, cell);
-        }
-        std::vector<int> comp_of_root((size_t)ncells, -1);
-        std::vector<std::vector<uint32_t>> members;
-        for (uint32_t i = 0; i < nrows; ++i) {
-            const int root = c->tune.col_split ? find(cr[i].c0) : 0;
-            if (comp_of_root[(size_t)root] < 0) { comp_of_root[(size_t)root] = (int)members.size(); members.emplace_back(); }
-            members[(size_t)comp_of_root[(size_t)root]].push_back(i);
-        }
-        std::vector<ColRow> sorted; sorted.reserve(nrows);
-        for (const auto& m : members) {
-            sar::ColumnComp cc{};
-            cc.group_first = (uint32_t)plan.group_begin.size(); cc.row_first = (uint32_t)sorted.size();
-            uint32_t last_round = never;
-            for (uint32_t i : m) {
-                if (cr[i].round != last_round) { plan.group_begin.push_back((uint32_t)sorted.size()); last_round = cr[i].round; }
-                sorted.push_back(cr[i]);
-            }
-            cc.group_end = (uint32_t)plan.group_begin.size(); cc.row_end = (uint32_t)sorted.size();
-            plan.max_comp_rows = std::max(plan.max_comp_rows, cc.row_end - cc.row_first);
-            plan.max_comp_groups = std::max(plan.max_comp_groups, cc.group_end - cc.group_first);
-            plan.comps.push_back(cc);
-        }
-        plan.group_begin.push_back((uint32_t)sorted.size());
-        cr.swap(sorted);
-    }
-
-    // Chunks that do not start on a 16-byte boundary (a buffer cut into a number of parts that its size was not
-    // padded for).  When all rows of a component start the same distance h in front of a boundary, on both sides,
-    // they are moved up to it and run as vectors; the h bytes in front are done element by element in the first
-    // column.  All rows of a component must move together: a column has to mean the same offsets in each of them.
-    for (const auto& cc : plan.comps) {
-        const uint32_t phase = (uint32_t)((uintptr_t)cr[cc.row_first].d.p0 & 15u), h = 16u - phase;
-        bool same = phase != 0 && phase % (uint32_t)es == 0;
-        for (uint32_t i = cc.row_first; i < cc.row_end && same; ++i) {
-            const sar::DevOp& d = cr[i].d;
-            same = d.kind != SAR_OP_MREDUCE && ((uintptr_t)d.p0 & 15u) == phase && ((uintptr_t)d.p1 & 15u) == phase && d.bytes > h;
-        }
-        if (!same) continue;
-        for (uint32_t i = cc.row_first; i < cc.row_end; ++i) {
-            sar::DevOp& d = cr[i].d;
-            d.p0 += h; d.p1 += h; d.bytes -= h;
-            d.flags |= sar::DEVOP_VEC | (h << sar::DEVOP_HEAD_SHIFT);
-        }
-    }
-    plan.widest_row = 0;
-    for (const auto& r : cr) plan.widest_row = std::max(plan.widest_row, r.d.bytes);
-
-    // column width: 512 vectors when that still leaves enough columns to fill the chip, else 256
-    plan.block = c->tune.col_block ? c->tune.col_block : (plan.widest_row / sar::column_bytes(512, false) >= 2048 ? 512 : 256);
-
-    // Latency plan: when the work items are so few that they are all resident at once, time goes into dependent
-    // round trips, not bandwidth, and nobody warms the scalar cache: a row read through scalar loads is a trip to
-    // L2.  A workgroup then copies the rows of its component into LDS first, and a lane moves one vector per row
-    // (few items are better spread over more workgroups).  Forwarding is kept only where it takes the loads out of
-    // most rows (see below).
-    {
-        const int lb = sar::column_latency_block();
-        const uint64_t lcols = (plan.widest_row + sar::column_bytes(lb, false) - 1) / sar::column_bytes(lb, false);
-        const uint64_t items = lcols * plan.comps.size();
-        const bool few = c->tune.col_latency_plan == 2 || (c->tune.col_latency_plan == 1 && items <= 8u * (uint64_t)std::max(1, c->cu_count));
-        if (few && (c->tune.col_block == 0 || c->tune.col_block == lb) &&
-            sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) <= sar::column_lds_budget()) {
-            plan.staged = true;
-            plan.block = lb;
-        }
-    }
-
-    // per cell, the rows that touch it, in order; a reducing row reads and writes its cell
-    struct Ev { uint32_t row; bool reads, writes; };
-    std::vector<std::vector<Ev>> ev((size_t)ncells);
-    for (uint32_t i = 0; i < nrows; ++i) {
-        if (cr[i].d.kind == SAR_OP_MREDUCE) {
-            for (int cell : cr[i].mreads)
-                ev[(size_t)cell].push_back({i, true, std::find(cr[i].mwrites.begin(), cr[i].mwrites.end(), cell) != cr[i].mwrites.end()});
-            for (int cell : cr[i].mwrites)
-                if (std::find(cr[i].mreads.begin(), cr[i].mreads.end(), cell) == cr[i].mreads.end()) ev[(size_t)cell].push_back({i, false, true});
-            continue;
-        }
-        const bool reduce = cr[i].d.kind != SAR_OP_COPY, both = cr[i].d.kind == SAR_OP_XREDUCE;
-        ev[(size_t)cr[i].c0].push_back({i, reduce, true});
-        if (cr[i].c1 != cr[i].c0) ev[(size_t)cr[i].c1].push_back({i, true, both});
-    }
-    // the next row after `i` that reads the cell's present value (never: it is overwritten first, or not read again)
-    auto next_read = [&](int cell, uint32_t i) {
-        const auto& v = ev[(size_t)cell];
-        auto it = std::upper_bound(v.begin(), v.end(), i, [](uint32_t x, const Ev& e) { return x < e.row; });
-        return (it != v.end() && it->reads) ? it->row : never;
-    };
-
-    // one pass of the slot bookkeeping with at most `max_slots` slots
-    struct Forwarding {
-        std::vector<uint32_t> flags, slots;      // per row: DEVOP_GET0 | GET1 | PUT and the packed slot numbers
-        uint32_t nslots = 0;
-        uint64_t bytes = 0;                      // operand bytes found in slots
-    };
-    auto forward = [&](uint32_t max_slots) {
-        Forwarding f;
-        f.flags.assign(nrows, 0); f.slots.assign(nrows, 0);
-        if (max_slots == 0) return f;
-        struct Slot { std::vector<int> cells; uint64_t bytes = 0; };
-        std::vector<Slot> slot(max_slots);
-        std::vector<int> cell_slot((size_t)ncells, -1);
-        auto drop_cell = [&](int cell) {
-            const int k = cell_slot[(size_t)cell];
-            if (k < 0) return;
-            auto& v = slot[(size_t)k].cells;
-            v.erase(std::remove(v.begin(), v.end(), cell), v.end());
-            cell_slot[(size_t)cell] = -1;
-        };
-        auto clear_slot = [&](int k) {
-            for (int cell : slot[(size_t)k].cells) cell_slot[(size_t)cell] = -1;
-            slot[(size_t)k].cells.clear();
-        };
-        auto slot_next_use = [&](int k, uint32_t i) {
-            uint32_t m = never;
-            for (int cell : slot[(size_t)k].cells) m = std::min(m, next_read(cell, i));
-            return m;
-        };
-        // a slot for a value next used at row `nu`: a free one, else the one whose own next use is furthest (and later than nu)
-        auto take_slot = [&](uint32_t nu, uint32_t i) {
-            int far = -1; uint32_t far_use = 0;
-            for (int k = 0; k < (int)max_slots; ++k) {
-                if (slot[(size_t)k].cells.empty()) return k;
-                const uint32_t u = slot_next_use(k, i);
-                if (u == never) { clear_slot(k); return k; }
-                if (u > far_use) { far_use = u; far = k; }
-            }
-            if (far >= 0 && far_use > nu) { clear_slot(far); return far; }
-            return -1;
-        };
-        for (uint32_t i = 0; i < nrows; ++i) {
-            const sar::DevOp& d = cr[i].d;
-            if (d.kind == SAR_OP_MREDUCE) {
-                // all operands come from memory (they are inputs nobody has touched); the result is a new value
-                uint32_t nu = never;
-                for (int cell : cr[i].mwrites) { drop_cell(cell); nu = std::min(nu, next_read(cell, i)); }
-                const int k = nu == never ? -1 : take_slot(nu, i);
-                if (k >= 0) {
-                    slot[(size_t)k].bytes = d.bytes;
-                    for (int cell : cr[i].mwrites) { slot[(size_t)k].cells.push_back(cell); cell_slot[(size_t)cell] = k; }
-                    f.flags[i] |= sar::DEVOP_PUT; f.slots[i] |= (uint32_t)k << 16;
-                    f.nslots = std::max(f.nslots, (uint32_t)k + 1);
-                }
-                continue;
-            }
-            const int c0 = cr[i].c0, c1 = cr[i].c1;
-            const bool reduce = d.kind != SAR_OP_COPY;
-            const bool can = (d.flags & sar::DEVOP_VEC) && c0 != c1;
-            int k0 = (can && reduce) ? cell_slot[(size_t)c0] : -1, k1 = can ? cell_slot[(size_t)c1] : -1;
-            if (k0 >= 0 && slot[(size_t)k0].bytes != d.bytes) k0 = -1;
-            if (k1 >= 0 && slot[(size_t)k1].bytes != d.bytes) k1 = -1;
-            if (k0 >= 0) { f.flags[i] |= sar::DEVOP_GET0; f.slots[i] |= (uint32_t)k0; f.bytes += d.bytes & ~(uint64_t)15u; f.nslots = std::max(f.nslots, (uint32_t)k0 + 1); }
-            if (k1 >= 0) { f.flags[i] |= sar::DEVOP_GET1; f.slots[i] |= (uint32_t)k1 << 8; f.bytes += d.bytes & ~(uint64_t)15u; f.nslots = std::max(f.nslots, (uint32_t)k1 + 1); }
-            // the row's result replaces what its destination cells held
-            drop_cell(c0);
-            if (d.kind == SAR_OP_XREDUCE) drop_cell(c1);
-            if (d.kind == SAR_OP_COPY && k1 >= 0) {
-                slot[(size_t)k1].cells.push_back(c0); cell_slot[(size_t)c0] = k1;          // the held value now lives in c0 too
-            } else if (can) {
-                uint32_t nu = next_read(c0, i);
-                if (d.kind != SAR_OP_REDUCE_INTO) nu = std::min(nu, next_read(c1, i));      // COPY: source and destination hold the value
-                const int k = nu == never ? -1 : take_slot(nu, i);
-                if (k >= 0) {
-                    if (d.kind == SAR_OP_COPY) drop_cell(c1);
-                    slot[(size_t)k].bytes = d.bytes;
-                    slot[(size_t)k].cells.push_back(c0); cell_slot[(size_t)c0] = k;
-                    if (d.kind != SAR_OP_REDUCE_INTO) { slot[(size_t)k].cells.push_back(c1); cell_slot[(size_t)c1] = k; }
-                    f.flags[i] |= sar::DEVOP_PUT; f.slots[i] |= (uint32_t)k << 16;
-                    f.nslots = std::max(f.nslots, (uint32_t)k + 1);
-                }
-            }
-        }
-        if (f.bytes == 0) { f.flags.assign(nrows, 0); f.slots.assign(nrows, 0); f.nslots = 0; }    // nothing found: no slots at all
-        return f;
-    };
-
-    Forwarding fwd = forward(0);
-    bool all_found = false;              // every re-read of the column finds its operand in a slot
-    if (c->tune.col_forward) {
-        const uint64_t table = plan.staged ? sar::column_table_bytes(plan.max_comp_rows, plan.max_comp_groups + 1) : 0u;
-        const uint32_t fit = (uint32_t)std::min<uint64_t>(255u, (sar::column_lds_budget() - table) / sar::column_bytes(plan.block, !plan.staged));
-        if (c->tune.col_slots > 0) {
-            fwd = forward(std::min<uint32_t>(fit, (uint32_t)c->tune.col_slots));
-            all_found = fwd.nslots && fwd.bytes == forward(255u).bytes;
-        } else {
-            // How many slots.  LDS per compute unit is what they cost: up to 5 per lane all 2048 lanes of a compute
-            // unit stay resident, up to 10 half of them.  Measured on MI355X, half occupancy pays when every re-read
-            // is then found in a slot (what still goes to memory is the cold inputs and the stores), but not for a
-            // part of them; and a plan that finds less than a tenth of the bytes the rows move is not worth the
-            // longer row loop.  (Component by component few values are alive at a time: one for the StragglAR
-            // tables and ring, four for halving-doubling at n = 8.)
-            const uint64_t all = forward(255u).bytes;
-            fwd = forward(std::min<uint32_t>(fit, 10u));
-            if (fwd.bytes != all) fwd = forward(std::min<uint32_t>(fit, 5u));
-            all_found = fwd.nslots && fwd.bytes == all;
-            uint64_t moved = 0;                  // algorithmic bytes of the rows
-            for (const auto& r : cr) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : r.d.kind == SAR_OP_MREDUCE ? r.d.nsrc + r.d.ndst : 3u);
-            if (fwd.bytes * 10u < moved) { fwd = forward(0); all_found = false; }
-            if (plan.staged && fwd.nslots) {
-                // Latency plan: the buffers sit in L2 and an operand from there arrives about as fast as one from a
-                // slot.  What forwarding buys is rows that load nothing at all (copies of a held value: no round trip
-                // in the chain).  Keep it when two thirds of the rows are such (the broadcast trees of the StragglAR
-                // tables and of direct: n = 32 at 1 MiB per rank 17.8 us against 21.8 us), not for chains whose
-                // rows mostly still load (ring, halving-doubling: 12.9 against 11.7 us at n = 8).
-                uint32_t free_rows = 0;
-                for (uint32_t i = 0; i < nrows; ++i) free_rows += cr[i].d.kind == SAR_OP_COPY && (fwd.flags[i] & sar::DEVOP_GET1);
-                if (free_rows * 3u < nrows * 2u) { fwd = forward(0); all_found = false; }
-            }
-        }
-    }
-    plan.nslots = fwd.nslots; plan.forwarded_bytes = fwd.bytes;
-
-    // Stores nobody needs.  A row's result for a cell is dead when a later row overwrites the cell and every row
-    // that reads it before then (the overwriting row included, if it reads) takes it from a slot: the partial
-    // sums of ring and halving-doubling, the pre-work's result ahead of the exchange in a same-launch run.  Only
-    // the whole vectors are left out; the bytes in front of the first and behind the last one always go through
-    // memory.  What the rank buffers hold after the launch does not change.
-    if (fwd.nslots && c->tune.col_elide_stores) {
-        auto from_slot = [&](uint32_t j, int cell) {            // does row j take the cell's value from a slot?
-            const sar::DevOp& d = cr[j].d;
-            if (d.kind == SAR_OP_MREDUCE || cr[j].c0 == cr[j].c1) return false;
-            if (cell == cr[j].c1) return (fwd.flags[j] & sar::DEVOP_GET1) != 0;
-            return cell == cr[j].c0 && d.kind != SAR_OP_COPY && (fwd.flags[j] & sar::DEVOP_GET0) != 0;
-        };
-        auto dead = [&](uint32_t i, int cell) {
-            if (!(cr[i].d.flags & sar::DEVOP_VEC)) return false;
-            const auto& v = ev[(size_t)cell];
-            for (auto it = std::upper_bound(v.begin(), v.end(), i, [](uint32_t x, const Ev& e) { return x < e.row; }); it != v.end(); ++it) {
-                if (it->reads && !from_slot(it->row, cell)) return false;
-                if (it->writes) return (cr[it->row].d.flags & sar::DEVOP_VEC) && cr[it->row].d.bytes == cr[i].d.bytes;
-            }
-            return false;                                       // never overwritten: part of the result
-        };
-        for (uint32_t i = 0; i < nrows; ++i) {
-            const sar::DevOp& d = cr[i].d;
-            const uint64_t vec_bytes = d.bytes & ~(uint64_t)15u;
-            if (d.kind == SAR_OP_MREDUCE) {
-                bool all = true;
-                for (int cell : cr[i].mwrites) all = all && dead(i, cell);
-                if (all) { fwd.flags[i] |= sar::DEVOP_DEAD0; plan.elided_bytes += vec_bytes * d.ndst; }
-                continue;
-            }
-            if (cr[i].c0 == cr[i].c1) continue;
-            if (dead(i, cr[i].c0)) { fwd.flags[i] |= sar::DEVOP_DEAD0; plan.elided_bytes += vec_bytes; }
-            if (d.kind == SAR_OP_XREDUCE && dead(i, cr[i].c1)) { fwd.flags[i] |= sar::DEVOP_DEAD1; plan.elided_bytes += vec_bytes; }
-        }
-    }
-    for (uint32_t i = 0; i < nrows; ++i) { cr[i].d.flags |= fwd.flags[i]; cr[i].d.slots = fwd.slots[i]; }
-
-    // Cache policy of the launch (the column kernel takes one for all its rows).  Planned (2): when every re-read is
-    // forwarded, what is still loaded is read exactly once: streaming loads (+1.5 % for the StragglAR table);
-    // otherwise the re-reads are meant to find their data in the caches and nothing streams (streaming loads cost
-    // 4-10 % there).  Streaming stores never paid in this kernel (-3 to -25 %).
-    plan.policy = c->tune.cache_policy == 0 ? 0u : c->tune.cache_policy == 1 ? 2u : c->tune.cache_policy == 3 ? 1u : (all_found ? 1u : 0u);
-
-    // Dispatch order of the items.  All columns of one component before the next component keeps the resident
-    // workgroups on few (rank, chunk) streams at a time (+3 to +5 % for the StragglAR tables, +2 % for ring at 64 MiB
-    // per rank and more).  It only matters, and only pays, when the items outnumber the resident workgroups
-    // severalfold and every row is vector-aligned; and it does not pay where a component reduces several pairs of
-    // ranks in the same round (halving-doubling: -4 to -15 %).  Otherwise the items of one column, all components,
-    // are dispatched together.
-    {
-        uint32_t most = 0;
-        bool aligned = true;
-        for (size_t g = 0; g + 1 < plan.group_begin.size(); ++g) {
-            uint32_t reducing = 0;
-            for (uint32_t i = plan.group_begin[g]; i < plan.group_begin[g + 1]; ++i) {
-                reducing += cr[i].d.kind != SAR_OP_COPY;
-                aligned &= (cr[i].d.flags & sar::DEVOP_VEC) != 0;
-            }
-            most = std::max(most, reducing);
-        }
-        const uint64_t cbytes = sar::column_bytes(plan.block, plan.nslots != 0 && !plan.staged);
-        const uint64_t items = (plan.widest_row + cbytes - 1) / cbytes * plan.comps.size();
-        const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (2048u / (uint32_t)plan.block);
-        plan.component_major = most <= 1 && aligned && !plan.staged && items >= 2 * resident;
-    }
-
-    plan.lane_local = true;
-    for (const auto& r : cr) {
-        if (!(r.d.flags & sar::DEVOP_VEC) || (r.d.bytes & 15u) || (r.d.flags >> sar::DEVOP_HEAD_SHIFT & 15u)) plan.lane_local = false;
-        rows.push_back(r.d);
-    }
-    return SAR_OK;
+int lower_column(const sar_ctx* c, const std::vector<const sar::Schedule*>& scheds, std::vector<sar::DevOp>& rows, std::vector<char*>& ptrs, ColumnPlan& plan) {
+    std::string error;
+    const int rc = sar::plan_columns(column_env(c), scheds, rows, ptrs, plan, &error);
+    return rc == SAR_OK ? SAR_OK : set_error(rc, error);
 }
 
 // Which executor is expected to be faster (executor = 2).  Constants are measurements on MI355X.
