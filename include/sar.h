@@ -150,7 +150,16 @@ uint64_t sar_pad_bytes(uint64_t bytes, int n);
 /* Parse a table in the text format the reference synthesizers print
  * (synthesizer_pow2.py:241-247, matching strings :54,:71,:84).  Closes the
  * reference's manual step "translate the output into ncclSend/ncclRecv by
- * hand" (README.md:35). */
+ * hand" (README.md:35).
+ * A text whose first line is "sar-rows <ranks> <parts>" is read as a row list
+ * instead, for schedules the matching strings cannot express: after a line
+ * "round", one row per line,
+ *   copy    <src_rank> <dst_rank> <src_chunk> <dst_chunk> [<nchunks>]
+ *   reduce  <src_rank> <dst_rank> <src_chunk> <dst_chunk> [<nchunks>]   (dst += src)
+ *   xreduce <rank_a> <rank_b> <chunk> [<nchunks>]                        (both get a + b)
+ * with '#' comments; chunks are size/parts elements.  Such a table is checked
+ * for ranges and for rows of one round that touch the same chunk of a rank
+ * with one of them writing, not for being an AllReduce. */
 int sar_schedule_parse(const char* text, size_t len, int n, sar_schedule** out);
 
 /* Built-in tables.  alg is one of

@@ -82,10 +82,73 @@ void parse_matching(const char* b, const char* e, int round, std::vector<Op>& ou
     if (s.p != s.end) fail("round " + std::to_string(round) + ": trailing text in matching '" + std::string(b, e) + "'");
 }
 
+// Row list: any schedule of chunk moves, one row per line.
+//   sar-rows <ranks> <parts>
+//   round
+//   copy <src_rank> <dst_rank> <src_chunk> <dst_chunk> [<nchunks>]
+//   reduce <src_rank> <dst_rank> <src_chunk> <dst_chunk> [<nchunks>]     dst += src
+//   xreduce <rank_a> <rank_b> <chunk> [<nchunks>]                         both sides get a + b
+// '#' starts a comment.  The buffer is cut into <parts> chunks of size/parts elements.
+Schedule parse_rows(const char* text, size_t len, int n) {
+    Schedule sch; sch.name = "rows";
+    const char* p = text; const char* end = text + len;
+    bool header = false;
+    int line_no = 0;
+    while (p < end) {
+        const char* eol = (const char*)std::memchr(p, '\n', (size_t)(end - p));
+        if (!eol) eol = end;
+        ++line_no;
+        const char* b = p; const char* e = eol;
+        if (const char* hash = (const char*)std::memchr(b, '#', (size_t)(e - b))) e = hash;
+        while (b < e && std::isspace((unsigned char)*b)) ++b;
+        while (e > b && std::isspace((unsigned char)e[-1])) --e;
+        p = eol < end ? eol + 1 : end;
+        if (b == e) continue;
+        Scanner s{b, e};
+        auto bad = [&](const std::string& why) { fail("line " + std::to_string(line_no) + ": " + why); };
+        auto done = [&]() { s.ws(); if (s.p != s.end) bad("trailing text"); };
+        if (!header) {
+            if (!(s.lit("sar-rows") && s.num(&sch.n) && s.num(&sch.parts))) bad("expected 'sar-rows <ranks> <parts>'");
+            done();
+            if (sch.n != n) bad("the table is for " + std::to_string(sch.n) + " ranks, not " + std::to_string(n));
+            if (sch.parts < 1) bad("parts must be positive");
+            header = true;
+            continue;
+        }
+        if (s.lit("round")) { done(); sch.rounds.emplace_back(); continue; }
+        if (sch.rounds.empty()) bad("a row before the first 'round' line");
+        int a = 0, d = 0, sc = 0, dc = 0, nch = 1;
+        if (s.lit("xreduce")) {
+            if (!(s.num(&a) && s.num(&d) && s.num(&sc))) bad("expected 'xreduce <rank_a> <rank_b> <chunk> [<nchunks>]'");
+            s.ws(); if (s.p != s.end && !s.num(&nch)) bad("malformed chunk count");
+            done();
+            sch.rounds.back().push_back(xreduce_op(a, d, sc, nch));
+            continue;
+        }
+        const bool is_copy = s.lit("copy");
+        if (!is_copy && !s.lit("reduce")) bad("unknown row '" + std::string(b, e) + "'");
+        if (!(s.num(&a) && s.num(&d) && s.num(&sc) && s.num(&dc))) bad("expected '<src_rank> <dst_rank> <src_chunk> <dst_chunk> [<nchunks>]'");
+        s.ws(); if (s.p != s.end && !s.num(&nch)) bad("malformed chunk count");
+        done();
+        sch.rounds.back().push_back(is_copy ? copy_op(a, d, sc, dc, nch) : reduce_into_op(a, d, sc, dc, nch));
+    }
+    if (!header) fail("no 'sar-rows' line");
+    if (sch.rounds.empty()) fail("no rounds found");
+    return sch;
+}
+
 }  // namespace
 
 Schedule parse_table(const char* text, size_t len, int n) {
     if (!text) fail("no text");
+    {
+        const char* b = text; const char* e = text + len;
+        while (b < e && std::isspace((unsigned char)*b)) ++b;
+        if ((size_t)(e - b) >= 8 && std::memcmp(b, "sar-rows", 8) == 0) {
+            if (n < 2 || n > SAR_MAX_RANKS) fail("n must be in [2, " + std::to_string(SAR_MAX_RANKS) + "]");
+            return parse_rows(text, len, n);
+        }
+    }
     if (n < 3 || n > SAR_MAX_RANKS) fail("n must be in [3, " + std::to_string(SAR_MAX_RANKS) + "]");
     Schedule sch; sch.n = n; sch.parts = n - 1; sch.stragglar_rules = true; sch.name = "stragglar";
     const char* p = text; const char* end = text + len;

@@ -34,7 +34,8 @@ struct Schedule {
 struct Range { uint64_t dst_off, src_off, len; };
 Range lower_range(const Schedule& s, const Op& op, uint64_t elems);
 
-// text format of the reference synthesizers -> schedule; throws std::runtime_error
+// text format of the reference synthesizers, or a row list (first line 'sar-rows <ranks> <parts>') -> schedule;
+// throws std::runtime_error
 Schedule parse_table(const char* text, size_t len, int n);
 Schedule builtin(const std::string& alg, int n);
 // empty string = valid, else the reason

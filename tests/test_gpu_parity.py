@@ -577,3 +577,86 @@ def test_segmented_execution(gpu_ctx, sarlib, oracle, alg):
         got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, None, delay=0.0, tuning=dict(executor=0, segments=seg))
         for r in range(n):
             assert_bits_equal(got[r], want[r], "%s segments=%d rank %d" % (alg, seg, r))
+
+
+def random_row_list(rng, n, parts, rounds):
+    """A random schedule as a row list: rows of one round never touch a chunk of a rank that another row of
+    the round writes.  Anything else goes: chunks change index on the way, ranges of several chunks, values
+    overwritten before or after they are read."""
+    lines, table = ["sar-rows %d %d" % (n, parts)], []
+    for _ in range(rounds):
+        lines.append("round")
+        reads, writes, rows = set(), set(), []
+        for _ in range(int(rng.integers(1, 2 * n))):
+            kind = ("copy", "reduce", "xreduce")[int(rng.integers(0, 3))]
+            a, b = (int(x) for x in rng.choice(n, 2, replace=False))
+            nch = int(rng.integers(1, min(3, parts) + 1))
+            sc, dc = int(rng.integers(0, parts - nch + 1)), int(rng.integers(0, parts - nch + 1))
+            if kind == "xreduce":
+                dc = sc
+            src = {(a, sc + k) for k in range(nch)}
+            dst = {(b, dc + k) for k in range(nch)}
+            r, w = (src | dst, src | dst) if kind == "xreduce" else (src | dst if kind == "reduce" else src, dst)
+            if (w & (reads | writes)) or (r & writes):
+                continue
+            reads |= r
+            writes |= w
+            rows.append((kind, a, b, sc, dc, nch))
+            lines.append("xreduce %d %d %d %d" % (a, b, sc, nch) if kind == "xreduce" else "%s %d %d %d %d %d" % (kind, a, b, sc, dc, nch))
+        table.append(rows)
+    return "\n".join(lines) + "\n", table
+
+
+def apply_row_list(oracle, table, bufs, parts, dtype):
+    """The rows on numpy arrays, in order (rows of one round do not depend on each other); the add is the
+    checker's orc_reduce_add."""
+    chunk = bufs[0].size // parts
+    for rows in table:
+        for kind, a, b, sc, dc, nch in rows:
+            src = bufs[a][sc * chunk:(sc + nch) * chunk]
+            dst = bufs[b][dc * chunk:(dc + nch) * chunk]
+            if kind == "copy":
+                dst[:] = src
+            elif kind == "reduce":
+                oracle.reduce_add(dst, src, dtype)                 # dst += src
+            else:
+                s = dst.copy()                                     # allreduce_8GPU.cu:564-578: both sides add the other's chunk
+                oracle.reduce_add(s, src, dtype)
+                dst[:] = s
+                src[:] = s
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_random_row_lists(gpu_ctx, sarlib, oracle, seed):
+    """Schedules nobody designed: random rows (copies, one-sided and two-sided reduces, across chunk indices, over
+    several chunks) through both executors and the planner's options, against the same rows applied with numpy and
+    the checker's add.  Exercises components that span chunk indices, values evicted from their slots, stores that
+    are and are not overwritten unread, and chunks off the vector boundary."""
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(2, 10))
+    parts = int(rng.integers(1, 7))
+    dtype = ("f32", "f16", "bf16")[seed % 3]
+    chunk_elems = int(rng.choice([1, 3, 4, 8, 37, 64, 257, 1024, 3000, 4096 + 4, 8192]))
+    elems = parts * chunk_elems + int(rng.integers(0, 3))
+    text, table = random_row_list(rng, n, parts, int(rng.integers(1, 11)))
+    main = sarlib.parse(text, n)
+    assert main.validate() == ""
+    inputs = make_inputs(n, elems, dtype, seed=seed, kind="ints" if seed % 2 else "normal", scale=2.0)
+    want = [x.copy() for x in inputs]
+    apply_row_list(oracle, table, want, parts, dtype)
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, elems * ES[dtype], dtype)
+    # (small buffers take the plan for few work items, which drops forwarding for most tables: asking for a number of
+    # slots keeps it)
+    for t in (dict(executor=1), dict(executor=0), dict(executor=1, col_forward=0), dict(executor=1, col_split=0, col_slots=3),
+              dict(executor=1, col_slots=2, col_elide_stores=0), dict(executor=1, col_latency_plan=0, col_slots=2),
+              dict(executor=1, col_latency_plan=0, col_slots=8), dict(executor=1, col_latency_plan=2, col_slots=1, col_wgs=1),
+              dict(executor=1, col_latency_plan=2, col_slots=5), dict(executor=1, col_latency_plan=0),
+              dict(executor=1, col_slots=4, col_light_sync=0, cache_policy=1, col_block=1024), dict(executor=2)):
+        ctx.set_tuning(**dict(ctx.default_tuning, **t))
+        for r, x in enumerate(inputs):
+            ctx.upload(r, x)
+        ctx.prepare(main, None, use_graph=bool(seed % 4 == 3))
+        ctx.run(-1.0)
+        for r in range(n):
+            assert_bits_equal(ctx.download(r), want[r], "seed %d n=%d parts=%d chunk %d %s tuning %r rank %d\n%s" % (seed, n, parts, chunk_elems, dtype, t, r, text))

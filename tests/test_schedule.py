@@ -217,6 +217,39 @@ def test_parser_errors(sarlib):
         sarlib.builtin("bogus", 8)
 
 
+def test_row_list_format(sarlib):
+    """The second text format of sar_schedule_parse: any rows, one per line.  The ring of
+    allreduce_8GPU.cu:146-198 written out as a row list must give the built-in ring's rows and bytes."""
+    import stragglar_amd as sa
+    n = 8
+    lines = ["sar-rows %d %d   # ring" % (n, n)]
+    for step in range(1, n):
+        lines.append("round")
+        lines += ["reduce %d %d %d %d" % ((r - 1) % n, r, (r - step - 1) % n, (r - step - 1) % n) for r in range(n)]
+    for step in range(0, n - 1):
+        lines.append("round   # all-gather step %d" % step)
+        lines += ["copy %d %d %d %d 1" % ((r - 1) % n, r, (r - step - 1) % n, (r - step - 1) % n) for r in range(n)]
+    mine, ring = sarlib.parse("\n".join(lines) + "\n", n), sarlib.builtin("ring", n)
+    assert mine.validate() == "" and (mine.ranks, mine.parts, mine.num_rounds) == (n, n, 2 * (n - 1))
+    assert [sorted(r) for r in mine.rounds()] == [sorted(r) for r in ring.rounds()]
+    assert mine.bytes(1 << 20, 4) == ring.bytes(1 << 20, 4)
+    # an exchange over two chunks, as halving-doubling's second step has it (allreduce_8GPU.cu:280-338)
+    x = sarlib.parse("sar-rows 4 4\nround\nxreduce 0 2 2 2\nreduce 1 3 0 1\n", 4)
+    assert x.validate() == ""
+    assert [(k, d, s_, dc, sc, nch) for (k, d, s_, dc, sc, nch, *_r) in x.rounds()[0]] == [(XREDUCE, 0, 2, 2, 2, 2), (REDUCE_INTO, 3, 1, 1, 0, 1)]
+    assert x.bytes(400, 4)[0] == 4 * 200 * 4 + 3 * 100 * 4
+    # what the validator still checks for such a table: ranges, and rows of a round that meet on a chunk one of them writes
+    assert "overlapping" in sarlib.parse("sar-rows 4 4\nround\ncopy 0 1 0 0\nreduce 1 2 0 0\n", 4).validate()
+    assert "out of range" in sarlib.parse("sar-rows 4 4\nround\ncopy 0 1 3 3 2\n", 4).validate()
+    assert "itself" in sarlib.parse("sar-rows 4 4\nround\ncopy 1 1 0 1\n", 4).validate()
+    for text in ["sar-rows 4 4\ncopy 0 1 0 0\n", "sar-rows 5 4\nround\ncopy 0 1 0 0\n", "sar-rows 4 4\nround\nmove 0 1 0 0\n",
+                 "sar-rows 4 4\nround\ncopy 0 1 0 0 1 7\n", "sar-rows 4 0\nround\n", "sar-rows 4 4\n", "sar-rows 4\nround\n",
+                 "sar-rows 4 4\nround\nxreduce 0 1\n"]:
+        with pytest.raises(sa.SarError) as ei:
+            sarlib.parse(text, 4)
+        assert ei.value.code == -5, text
+
+
 # ---- the package's own synthesizers against the reference's printed tables ------------------
 
 def golden_lists(name):
