@@ -51,7 +51,7 @@ public:
         if (fwd.nslots && env_.tune.col_elide_stores) mark_dead_stores(fwd);
         for (uint32_t i = 0; i < nrows(); ++i) { cr_[i].d.flags |= fwd.flags[i]; cr_[i].d.slots = fwd.slots[i]; }
         choose_launch();
-        for (const auto& r : cr_) rows.push_back(r.d);
+        for (const auto& r : cr_) { rows.push_back(r.d); plan_.multi_source |= r.d.kind == SAR_OP_MREDUCE; }
         return SAR_OK;
     }
 

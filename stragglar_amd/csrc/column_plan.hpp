@@ -47,6 +47,7 @@ struct ColumnPlan {
     bool staged = false;             // latency plan: a workgroup copies the rows of its component into LDS first
     uint32_t policy = 0;             // cache policy of the launch: 0 cached, 1 streaming loads, 2 streaming loads and stores
     bool unsupported = false;        // the rows cannot all run in the column kernel
+    bool multi_source = false;       // some rows are MREDUCE rows
     bool component_major = false;    // dispatch order of the items: all columns of a component, then the next component
 };
 

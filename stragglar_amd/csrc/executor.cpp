@@ -48,7 +48,7 @@ struct ColumnDevice {
     bool ready = false;
     uint32_t* d_group_begin = nullptr;
     sar::ColumnComp* d_comps = nullptr;
-    uint32_t first_op = 0, ncomp = 0, ncols = 0, run = 1, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0;
+    uint32_t first_op = 0, ncomp = 0, ncols = 0, run = 1, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0, multi_source = 0;
 };
 
 struct sar_ctx {
@@ -351,7 +351,7 @@ int launch_column_plan(sar_ctx* c, const ColumnDevice& d) {
     L.ops = c->d_ops + d.first_op; L.group_begin = d.d_group_begin; L.comps = d.d_comps; L.ptrs = c->d_ptrs;
     L.ncomp = d.ncomp; L.nitems = d.items;
     L.table_rows = d.table_rows; L.table_groups = d.table_groups;
-    L.lane_local = d.lane_local; L.policy = d.policy;
+    L.lane_local = d.lane_local; L.policy = d.policy; L.multi_source = d.multi_source;
     L.ncols = d.ncols; L.run = d.run;
     SAR_HIP(sar::launch_column(c->dtype, (int)d.block, d.grid, d.slots, c->stream, L));
     return SAR_OK;
@@ -370,6 +370,7 @@ int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, Colu
     d.block = (uint32_t)cp.block;
     d.slots = cp.nslots;
     d.lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
+    d.multi_source = cp.multi_source ? 1u : 0u;
     d.table_rows = cp.staged ? cp.max_comp_rows : 0u;
     d.table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
     d.policy = cp.policy;

@@ -397,7 +397,7 @@ static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offset
 // accesses cached, 1 = streaming (nontemporal) loads and cached stores, 2 = streaming loads and stores.  The
 // policy is a template argument because a flavour picked per row at run time does not survive compilation:
 // the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.
-template <int DT, int BLOCK, bool FWD, bool LAT, int POL>
+template <int DT, int BLOCK, bool FWD, bool LAT, int POL, bool MR>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
                                                         const ColumnComp* __restrict__ comps, char* const* __restrict__ ptrs, ColumnLaunch L) {
     typedef typename Elem<DT>::T T;
@@ -450,7 +450,7 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                 const uint64_t bytes = row.bytes;
                 char* const p0 = row.p0;
                 char* const p1 = row.p1;
-                if (kind == SAR_OP_MREDUCE) {
+                if (MR && kind == SAR_OP_MREDUCE) {
                     // Multi-source row (a pre-work collective lowered into the same launch; the host only does that
                     // when all its pointers are 16-byte aligned and the row is a whole number of vectors long):
                     // acc = srcs[0]; acc = srcs[k] + acc, the owner's own data last; the result goes to every dst
@@ -552,33 +552,33 @@ uint64_t column_lds_budget() { return 65536u; }
 uint64_t column_table_bytes(uint32_t rows, uint32_t groups) { return (uint64_t)rows * sizeof(DevOp) + (((uint64_t)groups + 3u) / 4u) * 16u; }
 int column_latency_block() { return 256; }
 
-template <int DT, bool FWD, int POL>
+template <int DT, bool FWD, int POL, bool MR>
 static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hipStream_t st, const ColumnLaunch& L) {
     switch (block) {
-        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
-        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
-        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL, MR>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL, MR>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL, MR>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-template <int DT, int POL>
+template <int DT, int POL, bool MR>
 static hipError_t launch_column_policy(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
     if (L.table_rows) {
-        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
-        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
+        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL, MR>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
+        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL, MR>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
         return hipGetLastError();
     }
-    return fwd ? launch_column_block<DT, true, POL>(block, grid, lds, st, L) : launch_column_block<DT, false, POL>(block, grid, lds, st, L);
+    return fwd ? launch_column_block<DT, true, POL, MR>(block, grid, lds, st, L) : launch_column_block<DT, false, POL, MR>(block, grid, lds, st, L);
 }
 
 template <int DT>
 static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
     switch (L.policy) {
-        case 0: return launch_column_policy<DT, 0>(block, grid, lds, fwd, st, L);
-        case 1: return launch_column_policy<DT, 1>(block, grid, lds, fwd, st, L);
-        case 2: return launch_column_policy<DT, 2>(block, grid, lds, fwd, st, L);
+        case 0: return L.multi_source ? launch_column_policy<DT, 0, true>(block, grid, lds, fwd, st, L) : launch_column_policy<DT, 0, false>(block, grid, lds, fwd, st, L);
+        case 1: return L.multi_source ? launch_column_policy<DT, 1, true>(block, grid, lds, fwd, st, L) : launch_column_policy<DT, 1, false>(block, grid, lds, fwd, st, L);
+        case 2: return L.multi_source ? launch_column_policy<DT, 2, true>(block, grid, lds, fwd, st, L) : launch_column_policy<DT, 2, false>(block, grid, lds, fwd, st, L);
         default: return hipErrorInvalidValue;
     }
 }

@@ -66,6 +66,7 @@ struct ColumnLaunch {
     uint32_t table_rows;         // 0, or the most rows of a component: latency plan, the workgroup copies the rows and
     uint32_t table_groups;       // group boundaries (at most table_groups) of its component into LDS first (block =
                                  // column_latency_block())
+    uint32_t multi_source;       // != 0: some rows are MREDUCE rows (a kernel variant of its own: their loads cost registers)
     uint32_t lane_local;         // != 0 promises that no lane reads bytes another lane wrote (all rows 16-byte
                                  // aligned, no partial vectors): groups are then separated by an execution barrier only
     uint32_t policy;             // whole launch: 0 = cached accesses, 1 = streaming loads, 2 = streaming loads and stores
