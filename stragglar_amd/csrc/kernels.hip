@@ -463,12 +463,12 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                         const uint64_t o = voff + v * vstep;
                         if (o + 16u <= bytes) {
                             f4 acc = ld16<LNT>(srcs[0] + o);
-                            for (uint32_t k0 = 1; k0 < row.nsrc; k0 += 8u) {
-                                f4 t[8];
+                            for (uint32_t k0 = 1; k0 < row.nsrc; k0 += 4u) {
+                                f4 t[4];
 #pragma unroll
-                                for (uint32_t q = 0; q < 8u; ++q) if (k0 + q < row.nsrc) t[q] = ld16<LNT>(srcs[k0 + q] + o);
+                                for (uint32_t q = 0; q < 4u; ++q) if (k0 + q < row.nsrc) t[q] = ld16<LNT>(srcs[k0 + q] + o);
 #pragma unroll
-                                for (uint32_t q = 0; q < 8u; ++q) if (k0 + q < row.nsrc) acc = add16<DT>(t[q], acc);
+                                for (uint32_t q = 0; q < 4u; ++q) if (k0 + q < row.nsrc) acc = add16<DT>(t[q], acc);
                             }
                             if (!(FWD && (flags & DEVOP_DEAD0))) for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(dsts[d] + o, acc);
                             if (FWD && (flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = acc;
