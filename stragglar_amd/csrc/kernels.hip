@@ -350,14 +350,15 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // Rows move whole chunks, so an element only ever meets the elements at its own offset within a
 // chunk: the schedule falls apart into independent "columns" (one range of within-chunk offsets each).
 // A workgroup owns a column of BLOCK 16-byte vectors and walks ALL rounds for it, row after row, with
-// nothing but a workgroup barrier between rounds.  Every row performs its stores on the rank buffers,
-// in schedule order for each element.  What a later round re-reads was written by the same lane moments
-// ago: without forwarding it comes back from L2 / Infinity Cache instead of HBM; with forwarding (FWD)
-// the lane kept it in an LDS value slot that the host assigned when it lowered the schedule, and the
-// load is not issued at all.
-// One row at a time and one vector per lane turned out best (32-38 VGPRs, eight waves per SIMD
-// resident: the other workgroups of the compute unit cover a row's latency; batching the loads of
-// several rows or several vectors per lane cost occupancy and was slower: 6.8 against 7.1 TB/s).
+// nothing but a workgroup barrier between rounds.  What a later round re-reads was written by the same
+// lane moments ago: without forwarding it comes back from L2 / Infinity Cache instead of HBM; with
+// forwarding (FWD) the lane kept it in an LDS value slot that the host assigned when it lowered the
+// schedule, and the load is not issued at all.  Every row stores its result to the rank buffers, in
+// schedule order for each element, except where the host found that a later row overwrites the value
+// before anybody loads it (DEVOP_DEAD0 / DEAD1).
+// One row at a time turned out best (24 VGPRs without forwarding, 48 with: eight waves per SIMD
+// resident, the other workgroups of the compute unit cover a row's latency; batching the loads of
+// several rows cost occupancy and was slower: 6.8 against 7.1 TB/s).
 
 // One row as the column kernel uses it, every field wave-uniform (SGPRs).
 struct ColRow { char* p0; char* p1; uint64_t bytes; uint32_t kind, flags, slots, nsrc, ndst, ptr_off; };
@@ -396,7 +397,9 @@ static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offset
 // groups of the item's component are copied into LDS first.  POL: cache policy of the whole launch, 0 = all
 // accesses cached, 1 = streaming (nontemporal) loads and cached stores, 2 = streaming loads and stores.  The
 // policy is a template argument because a flavour picked per row at run time does not survive compilation:
-// the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.
+// the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.  MR: the
+// launch has multi-source rows (a pre-work collective in the same launch); their batched loads double the
+// register count, so launches without such rows run a variant without that path.
 template <int DT, int BLOCK, bool FWD, bool LAT, int POL, bool MR>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
                                                         const ColumnComp* __restrict__ comps, char* const* __restrict__ ptrs, ColumnLaunch L) {
