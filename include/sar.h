@@ -286,6 +286,43 @@ int sar_default_tuning(sar_tuning_t* out);
 int sar_plan(const sar_schedule* prework, const sar_schedule* main_schedule, int n, uint64_t bytes_per_rank, int dtype,
              const sar_tuning_t* tuning, int compute_units, sar_stats_t* out);
 
+/* One row of the column executor's plan, as sar_plan_rows() reports it.  A work item of the kernel is one
+ * component for one column (a range of within-chunk offsets); it walks the component's rows in this order. */
+typedef struct sar_plan_row {
+    int32_t kind;        /* SAR_OP_*                                                                           */
+    int32_t component;   /* rows of different components never touch the same chunk of a rank                   */
+    int32_t group;       /* rows of one component and round; the workgroup meets at a barrier after each group  */
+    int32_t vector;      /* 1 = runs as 16-byte vectors, 0 = element by element                                 */
+    int32_t dst_rank;    /* rank of p0 (COPY/REDUCE_INTO: destination; XREDUCE: first side; MREDUCE: -1)        */
+    int32_t src_rank;    /* rank of p1 (source / second side; MREDUCE: -1)                                      */
+    uint64_t dst_off;    /* byte offset in dst_rank's buffer of the row's first whole vector                    */
+    uint64_t src_off;    /* the same for src_rank                                                               */
+    uint64_t bytes;      /* length from there                                                                   */
+    int32_t head_bytes;  /* bytes of the row in front of dst_off / src_off (a chunk that starts off the 16-byte */
+                         /* boundary): done element by element in the first column                              */
+    int32_t get0_slot;   /* value slot the operand at p0 is taken from instead of being loaded, -1 = loaded     */
+    int32_t get1_slot;   /* the same for the operand at p1                                                      */
+    int32_t put_slot;    /* value slot the result is kept in, -1 = not kept                                     */
+    int32_t dead0;       /* 1 = the whole vectors of the result are not stored to p0 (MREDUCE: to any           */
+                         /* destination): a later row overwrites them before anybody loads them                 */
+    int32_t dead1;       /* the same for p1 (XREDUCE)                                                           */
+    int32_t nsrc;        /* MREDUCE: sources, in add order ...                                                  */
+    int32_t ndst;        /* ... and destinations: entries [first_ptr, first_ptr + nsrc + ndst) of the pointer   */
+    int32_t first_ptr;   /* list                                                                                */
+    int32_t reserved;
+} sar_plan_row;
+
+typedef struct sar_plan_ptr { int32_t rank; int32_t reserved; uint64_t off; } sar_plan_ptr;
+
+/* The rows behind sar_plan(): the column executor's plan for the main schedule (same_launch 0) or for pre-work
+ * and main schedule in one launch (same_launch 1), whether or not the cost model would pick that executor.
+ * Writes at most row_cap rows and ptr_cap pointer-list entries; *nrows and *nptrs are the full counts.
+ * SAR_ESTATE when there is no such plan (executor 0, rows the column kernel cannot run, no pre-work).
+ * Host only; for tools and for tests that check the plan row by row. */
+int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_schedule, int n, uint64_t bytes_per_rank, int dtype,
+                  const sar_tuning_t* tuning, int compute_units, int same_launch,
+                  sar_plan_row* rows, int row_cap, int* nrows, sar_plan_ptr* ptrs, int ptr_cap, int* nptrs);
+
 #ifdef __cplusplus
 }
 #endif

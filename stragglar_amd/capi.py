@@ -45,6 +45,19 @@ class Stats(ctypes.Structure):
                 ("elided_store_bytes", ctypes.c_uint64)]
 
 
+class PlanRow(ctypes.Structure):
+    """sar_plan_row: one row of the column executor's plan."""
+    _fields_ = [("kind", ctypes.c_int32), ("component", ctypes.c_int32), ("group", ctypes.c_int32), ("vector", ctypes.c_int32),
+                ("dst_rank", ctypes.c_int32), ("src_rank", ctypes.c_int32), ("dst_off", ctypes.c_uint64), ("src_off", ctypes.c_uint64),
+                ("bytes", ctypes.c_uint64), ("head_bytes", ctypes.c_int32), ("get0_slot", ctypes.c_int32), ("get1_slot", ctypes.c_int32),
+                ("put_slot", ctypes.c_int32), ("dead0", ctypes.c_int32), ("dead1", ctypes.c_int32), ("nsrc", ctypes.c_int32),
+                ("ndst", ctypes.c_int32), ("first_ptr", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
+class PlanPtr(ctypes.Structure):
+    _fields_ = [("rank", ctypes.c_int32), ("reserved", ctypes.c_int32), ("off", ctypes.c_uint64)]
+
+
 class Tuning(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd", "segments",
                                                  "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores")]
@@ -71,7 +84,7 @@ EXPORTS = [
     "sar_create", "sar_destroy", "sar_alloc_ranks", "sar_adopt_ranks", "sar_upload", "sar_download", "sar_fill_const",
     "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
-    "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_default_tuning",
+    "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
 ]
 
 
@@ -124,6 +137,7 @@ class Library:
             "sar_sleep_ticks": (c_int, [vp, ctypes.c_float, P(ctypes.c_int64)]),
             "sar_stats": (c_int, [vp, P(Stats)]),
             "sar_plan": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, P(Stats)]),
+            "sar_plan_rows": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, c_int, P(PlanRow), c_int, P(c_int), P(PlanPtr), c_int, P(c_int)]),
             "sar_default_tuning": (c_int, [P(Tuning)]),
         }
         assert sorted(sig) == sorted(EXPORTS)
@@ -161,6 +175,22 @@ class Library:
         self.check(self.lib.sar_plan(prework.handle if prework else None, main.handle, n, bytes_per_rank, DTYPES[dtype],
                                      ctypes.byref(t), compute_units, ctypes.byref(st)))
         return st
+
+    def plan_rows(self, main: "Schedule", n: int, bytes_per_rank: int, dtype: str = "f32", prework: Optional["Schedule"] = None,
+                  same_launch: bool = False, compute_units: int = 0, **tuning):
+        """The rows of the column executor's plan and the pointer lists of its multi-source rows (as (rank, byte
+        offset) pairs): what ``plan`` summarises, row by row."""
+        t = self.default_tuning()
+        for k, v in tuning.items():
+            if not hasattr(t, k):
+                raise KeyError(k)
+            setattr(t, k, v)
+        nrows, nptrs = ctypes.c_int(0), ctypes.c_int(0)
+        args = (prework.handle if prework else None, main.handle, n, bytes_per_rank, DTYPES[dtype], ctypes.byref(t), compute_units, int(same_launch))
+        self.check(self.lib.sar_plan_rows(*args, None, 0, ctypes.byref(nrows), None, 0, ctypes.byref(nptrs)))
+        rows, ptrs = (PlanRow * max(1, nrows.value))(), (PlanPtr * max(1, nptrs.value))()
+        self.check(self.lib.sar_plan_rows(*args, rows, nrows.value, ctypes.byref(nrows), ptrs, nptrs.value, ctypes.byref(nptrs)))
+        return list(rows)[:nrows.value], [(p.rank, p.off) for p in list(ptrs)[:nptrs.value]]
 
     def parse(self, text: str, n: int) -> "Schedule":
         raw = text.encode()

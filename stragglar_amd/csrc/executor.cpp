@@ -462,6 +462,38 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_elide_stores == 0 || t.col_elide_stores == 1);
 }
 
+// sar_plan / sar_plan_rows: a context that never touches the device, with the rank buffers at made-up, suitably
+// aligned addresses (only ever used for arithmetic), and everything sar_prepare would decide for it.
+struct HostPlan {
+    sar_ctx c;
+    uint64_t stride = 0;
+    std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
+    ColumnPlan cp, fp;
+    uint32_t col_first = 0, fused_first = 0;
+    bool want_column = false, want_fused = false;
+
+    int make(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+             const sar_tuning_t* tuning, int compute_units) {
+        if (!main_sched) return set_error(SAR_EINVAL, "null argument");
+        if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
+        if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
+        if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+        if (tuning && !valid_tuning(*tuning)) return set_error(SAR_EINVAL, "tuning value out of range");
+        for (const sar_schedule* s : {prework, main_sched}) {
+            if (!s) continue;
+            if (s->s.n != n) return set_error(SAR_EINVAL, "schedule and rank count disagree");
+            std::string why = sar::validate(s->s);
+            if (!why.empty()) return set_error(SAR_ESCHED, why);
+        }
+        c.n = n; c.dtype = dtype; c.bytes_per_rank = bytes_per_rank;
+        c.cu_count = compute_units > 0 ? compute_units : 256;
+        if (tuning) c.tune = *tuning;
+        stride = (bytes_per_rank + (2u << 20) - 1) & ~(uint64_t)((2u << 20) - 1);
+        for (int r = 0; r < n; ++r) c.adopted.push_back(reinterpret_cast<char*>((uintptr_t)1 << 40) + (uint64_t)r * stride);
+        return plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused);
+    }
+};
+
 }  // namespace
 
 extern "C" {
@@ -900,30 +932,56 @@ int sar_default_tuning(sar_tuning_t* out) {
 
 int sar_plan(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
              const sar_tuning_t* tuning, int compute_units, sar_stats_t* out) {
-    if (!main_sched || !out) return set_error(SAR_EINVAL, "null argument");
-    if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
-    if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
-    if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
-    if (tuning && !valid_tuning(*tuning)) return set_error(SAR_EINVAL, "tuning value out of range");
-    for (const sar_schedule* s : {prework, main_sched}) {
-        if (!s) continue;
-        if (s->s.n != n) return set_error(SAR_EINVAL, "schedule and rank count disagree");
-        std::string why = sar::validate(s->s);
-        if (!why.empty()) return set_error(SAR_ESCHED, why);
-    }
-    // a context that never touches the device: rank buffers at made-up, suitably aligned addresses (only ever
-    // used for arithmetic here)
-    sar_ctx c;
-    c.n = n; c.dtype = dtype; c.bytes_per_rank = bytes_per_rank;
-    c.cu_count = compute_units > 0 ? compute_units : 256;
-    if (tuning) c.tune = *tuning;
-    const uint64_t stride = (bytes_per_rank + (2u << 20) - 1) & ~(uint64_t)((2u << 20) - 1);
-    for (int r = 0; r < n; ++r) c.adopted.push_back(reinterpret_cast<char*>((uintptr_t)1 << 40) + (uint64_t)r * stride);
-    std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    ColumnPlan cp, fp; uint32_t col_first = 0, fused_first = 0; bool want_column = false, want_fused = false;
-    int rc = plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused);
+    if (!out) return set_error(SAR_EINVAL, "null argument");
+    HostPlan hp;
+    const int rc = hp.make(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units);
     if (rc != SAR_OK) return rc;
-    *out = plan_stats(&c, prework, main_sched, cp, want_column, want_column && want_fused);
+    *out = plan_stats(&hp.c, prework, main_sched, hp.cp, hp.want_column, hp.want_column && hp.want_fused);
+    return SAR_OK;
+}
+
+int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+                  const sar_tuning_t* tuning, int compute_units, int same_launch,
+                  sar_plan_row* out_rows, int row_cap, int* nrows, sar_plan_ptr* out_ptrs, int ptr_cap, int* nptrs) {
+    if (!nrows || !nptrs || (row_cap > 0 && !out_rows) || (ptr_cap > 0 && !out_ptrs) || row_cap < 0 || ptr_cap < 0)
+        return set_error(SAR_EINVAL, "null argument");
+    HostPlan hp;
+    const int rc = hp.make(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units);
+    if (rc != SAR_OK) return rc;
+    const ColumnPlan& cp = same_launch ? hp.fp : hp.cp;
+    const size_t first = same_launch ? hp.fused_first : hp.col_first;
+    const size_t count = cp.group_begin.empty() ? 0 : cp.group_begin.back();
+    if (cp.unsupported || count == 0 || first + count > hp.rows.size())
+        return set_error(SAR_ESTATE, same_launch ? "no plan for pre-work and schedule in one launch" : "no column plan for this schedule and tuning");
+    auto locate = [&](const char* p, int32_t* rank, uint64_t* off) {
+        const uint64_t d = (uint64_t)(p - hp.c.adopted[0]);
+        *rank = (int32_t)(d / hp.stride); *off = d % hp.stride;
+    };
+    *nrows = (int)count; *nptrs = (int)hp.ptrs.size();
+    for (size_t k = 0; k < hp.ptrs.size() && k < (size_t)ptr_cap; ++k) { out_ptrs[k] = sar_plan_ptr{}; locate(hp.ptrs[k], &out_ptrs[k].rank, &out_ptrs[k].off); }
+    for (size_t comp = 0; comp < cp.comps.size(); ++comp) {
+        for (uint32_t g = cp.comps[comp].group_first; g < cp.comps[comp].group_end; ++g) {
+            for (uint32_t i = cp.group_begin[g]; i < cp.group_begin[g + 1] && i < (uint32_t)row_cap; ++i) {
+                const sar::DevOp& d = hp.rows[first + i];
+                sar_plan_row r{};
+                r.kind = (int32_t)d.kind; r.component = (int32_t)comp; r.group = (int32_t)(g - cp.comps[comp].group_first);
+                r.vector = (d.flags & sar::DEVOP_VEC) ? 1 : 0;
+                r.bytes = d.bytes; r.head_bytes = (int32_t)(d.flags >> sar::DEVOP_HEAD_SHIFT & 15u);
+                r.get0_slot = (d.flags & sar::DEVOP_GET0) ? (int32_t)(d.slots & 0xffu) : -1;
+                r.get1_slot = (d.flags & sar::DEVOP_GET1) ? (int32_t)(d.slots >> 8 & 0xffu) : -1;
+                r.put_slot = (d.flags & sar::DEVOP_PUT) ? (int32_t)(d.slots >> 16 & 0xffu) : -1;
+                r.dead0 = (d.flags & sar::DEVOP_DEAD0) ? 1 : 0; r.dead1 = (d.flags & sar::DEVOP_DEAD1) ? 1 : 0;
+                if (d.kind == SAR_OP_MREDUCE) {
+                    r.dst_rank = r.src_rank = -1;
+                    r.nsrc = (int32_t)d.nsrc; r.ndst = (int32_t)d.ndst; r.first_ptr = (int32_t)d.ptr_off;
+                } else {
+                    locate(d.p0, &r.dst_rank, &r.dst_off);
+                    locate(d.p1, &r.src_rank, &r.src_off);
+                }
+                out_rows[i] = r;
+            }
+        }
+    }
     return SAR_OK;
 }
 

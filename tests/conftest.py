@@ -79,3 +79,50 @@ def assert_bits_equal(got, want, what=""):
         i = int(np.flatnonzero(bad)[0])
         raise AssertionError("%s: %d of %d elements differ, first at %d: got %r want %r"
                              % (what, int(bad.sum()), bad.size, i, got[i], want[i]))
+
+
+def random_row_list(rng, n, parts, rounds):
+    """A random schedule as a row list: rows of one round never touch a chunk of a rank that another row of
+    the round writes.  Anything else goes: chunks change index on the way, ranges of several chunks, values
+    overwritten before or after they are read."""
+    lines, table = ["sar-rows %d %d" % (n, parts)], []
+    for _ in range(rounds):
+        lines.append("round")
+        reads, writes, rows = set(), set(), []
+        for _ in range(int(rng.integers(1, 2 * n))):
+            kind = ("copy", "reduce", "xreduce")[int(rng.integers(0, 3))]
+            a, b = (int(x) for x in rng.choice(n, 2, replace=False))
+            nch = int(rng.integers(1, min(3, parts) + 1))
+            sc, dc = int(rng.integers(0, parts - nch + 1)), int(rng.integers(0, parts - nch + 1))
+            if kind == "xreduce":
+                dc = sc
+            src = {(a, sc + k) for k in range(nch)}
+            dst = {(b, dc + k) for k in range(nch)}
+            r, w = (src | dst, src | dst) if kind == "xreduce" else (src | dst if kind == "reduce" else src, dst)
+            if (w & (reads | writes)) or (r & writes):
+                continue
+            reads |= r
+            writes |= w
+            rows.append((kind, a, b, sc, dc, nch))
+            lines.append("xreduce %d %d %d %d" % (a, b, sc, nch) if kind == "xreduce" else "%s %d %d %d %d %d" % (kind, a, b, sc, dc, nch))
+        table.append(rows)
+    return "\n".join(lines) + "\n", table
+
+
+def apply_row_list(oracle, table, bufs, parts, dtype):
+    """The rows on numpy arrays, in order (rows of one round do not depend on each other); the add is the
+    checker's orc_reduce_add."""
+    chunk = bufs[0].size // parts
+    for rows in table:
+        for kind, a, b, sc, dc, nch in rows:
+            src = bufs[a][sc * chunk:(sc + nch) * chunk]
+            dst = bufs[b][dc * chunk:(dc + nch) * chunk]
+            if kind == "copy":
+                dst[:] = src
+            elif kind == "reduce":
+                oracle.reduce_add(dst, src, dtype)                 # dst += src
+            else:
+                s = dst.copy()                                     # allreduce_8GPU.cu:564-578: both sides add the other's chunk
+                oracle.reduce_add(s, src, dtype)
+                dst[:] = s
+                src[:] = s

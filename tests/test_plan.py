@@ -137,3 +137,155 @@ def test_chunks_off_the_vector_boundary_are_still_forwarded(sarlib):
     heads = [(16 - (c * chunk) % 16) % 16 for c in range(6)]
     tails = [(chunk - h) % 16 for h in heads]
     assert ring.forwarded_bytes == 9 * (6 * chunk - sum(heads) - sum(tails))     # 4 of 5 reduce-scatter reads + 5 all-gather copies per chunk
+
+
+# ---- the plan, row by row, carried out on the CPU -------------------------------------------------------------
+# sar_plan_rows reports what the column kernel would be told.  Carrying those rows out with numpy - operands
+# from value slots where the plan says so, stores left out where it says they are dead, the bytes in front of
+# and behind the whole vectors through memory - must give the buffers the checker computes from the schedule.
+
+ES = {"f32": 4, "f16": 2, "bf16": 2}
+
+
+def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
+    es = ES[dtype]
+    slots = {}
+
+    def view(rank, lo, hi):
+        assert lo % es == 0 and hi % es == 0 and 0 <= lo <= hi <= bufs[rank].size * es
+        return bufs[rank][lo // es:hi // es]
+
+    def through_memory(r, lo_d, lo_s, nbytes):
+        if nbytes == 0:
+            return
+        dst, src = view(r.dst_rank, lo_d, lo_d + nbytes), view(r.src_rank, lo_s, lo_s + nbytes)
+        if r.kind == 0:
+            dst[:] = src
+        elif r.kind == 2:
+            oracle.reduce_add(dst, src, dtype)
+        else:
+            oracle.reduce_add(dst, src, dtype)
+            src[:] = dst
+
+    last = (-1, -1)
+    for r in rows:
+        assert (r.component, r.group) >= last, "rows come component by component, group by group"
+        last = (r.component, r.group)
+        if r.kind == 3:
+            assert r.vector and r.bytes % 16 == 0 and r.head_bytes == 0
+            srcs, dsts = ptrs[r.first_ptr:r.first_ptr + r.nsrc], ptrs[r.first_ptr + r.nsrc:r.first_ptr + r.nsrc + r.ndst]
+            acc = view(srcs[0][0], srcs[0][1], srcs[0][1] + r.bytes).copy()
+            for rank, off in srcs[1:]:
+                t = view(rank, off, off + r.bytes).copy()
+                oracle.reduce_add(t, acc, dtype)                 # the next source + what has been summed so far
+                acc = t
+            if not r.dead0:
+                for rank, off in dsts:
+                    view(rank, off, off + r.bytes)[:] = acc
+            if r.put_slot >= 0:
+                slots[(r.component, r.put_slot)] = acc
+            continue
+        if not r.vector:
+            assert r.head_bytes == 0 and r.get0_slot < 0 and r.get1_slot < 0 and r.put_slot < 0 and not r.dead0 and not r.dead1
+            through_memory(r, r.dst_off, r.src_off, r.bytes)
+            continue
+        assert r.dst_off % 16 == 0 and r.src_off % 16 == 0
+        vec = r.bytes & ~15
+        through_memory(r, r.dst_off - r.head_bytes, r.src_off - r.head_bytes, r.head_bytes)
+        through_memory(r, r.dst_off + vec, r.src_off + vec, r.bytes - vec)
+        dst, src = view(r.dst_rank, r.dst_off, r.dst_off + vec), view(r.src_rank, r.src_off, r.src_off + vec)
+        b = slots[(r.component, r.get1_slot)] if r.get1_slot >= 0 else src.copy()
+        assert b.size == dst.size, "a slot holds a value of another length"
+        if r.kind == 0:
+            assert r.get0_slot < 0
+            s = b
+        else:
+            s = (slots[(r.component, r.get0_slot)] if r.get0_slot >= 0 else dst).copy()
+            assert s.size == dst.size
+            oracle.reduce_add(s, b, dtype)
+        if not r.dead0:
+            dst[:] = s
+        if r.kind == 1 and not r.dead1:
+            src[:] = s
+        assert r.kind == 1 or not r.dead1
+        if r.put_slot >= 0:
+            slots[(r.component, r.put_slot)] = s.copy()
+
+
+PLAN_SETTINGS = [dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_slots=1), dict(col_latency_plan=0, col_slots=3),
+                 dict(col_latency_plan=2, col_slots=8), dict(col_forward=0), dict(col_split=0, col_slots=4), dict(col_latency_plan=0, col_elide_stores=0)]
+
+
+@pytest.mark.parametrize("dtype,chunk_elems", [("f32", 1024), ("f32", 4 * 37 + 1), ("bf16", 8 * 50), ("f16", 8 * 21 + 3)])
+@pytest.mark.parametrize("alg,n", [("stragglar", 8), ("stragglar", 4), ("ring", 8), ("ring", 5), ("rhd", 8), ("direct", 8), ("stragglar", 16)])
+def test_plans_of_the_four_algorithms_carried_out_on_the_cpu(sarlib, oracle, alg, n, dtype, chunk_elems):
+    from conftest import assert_bits_equal, make_inputs
+    table = {4: "stragglar_n4_cu.txt", 8: "stragglar_n8_cu.txt", 16: "synth_pow2_n16.txt"}.get(n) if alg == "stragglar" else None
+    main = sarlib.parse(read_golden(table), n) if table else sarlib.builtin(alg, n)
+    elems = main.parts * chunk_elems + (2 if main.parts > 1 else 0)
+    inputs = make_inputs(n, elems, dtype, seed=3, kind="normal", scale=2.0)
+    from oracle import parse_table
+    want = [x.copy() for x in inputs]
+    oracle.run(alg, want, dtype, rounds=parse_table(read_golden(table)) if table else None, delay=-1.0)
+    for t in PLAN_SETTINGS:
+        rows, ptrs = sarlib.plan_rows(main, n, elems * ES[dtype], dtype, executor=1, **t)
+        got = [x.copy() for x in inputs]
+        carry_out_plan(oracle, rows, ptrs, got, dtype)
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s n=%d %s chunk %d settings %r rank %d" % (alg, n, dtype, chunk_elems, t, r))
+
+
+@pytest.mark.parametrize("n,table", [(4, "stragglar_n4_cu.txt"), (6, "synth_nonpow2_n6.txt"), (8, "synth_pow2_n8.txt"), (12, "synth_nonpow2_n12.txt")])
+def test_plan_with_the_prework_in_the_same_launch_carried_out_on_the_cpu(sarlib, oracle, n, table):
+    from conftest import assert_bits_equal, make_inputs
+    from oracle import parse_table
+    main, pre = sarlib.parse(read_golden(table), n), sarlib.builtin("prework_rs", n)
+    for dtype, chunk_elems in (("f32", 256), ("f16", 8 * 33)):
+        elems = (n - 1) * chunk_elems
+        inputs = make_inputs(n, elems, dtype, seed=4)
+        want = [x.copy() for x in inputs]
+        oracle.run("stragglar", want, dtype, rounds=parse_table(read_golden(table)), delay=0.0)
+        for t in (dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_elide_stores=0), dict(col_forward=0)):
+            rows, ptrs = sarlib.plan_rows(main, n, elems * ES[dtype], dtype, prework=pre, same_launch=True, executor=1, **t)
+            assert sum(r.kind == 3 for r in rows) == n - 1
+            if t.get("col_latency_plan") == 0 and t.get("col_elide_stores", 1):
+                # (bandwidth plan, forwarding on) the pre-work's result goes to the exchange in a slot and is overwritten by it: never stored
+                assert all(r.dead0 and r.put_slot >= 0 for r in rows if r.kind == 3)
+            got = [x.copy() for x in inputs]
+            carry_out_plan(oracle, rows, ptrs, got, dtype)
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "n=%d %s settings %r rank %d" % (n, dtype, t, r))
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_plans_of_random_row_lists_carried_out_on_the_cpu(sarlib, oracle, seed):
+    import numpy as np
+    from conftest import apply_row_list, assert_bits_equal, make_inputs, random_row_list
+    rng = np.random.default_rng(7000 + seed)
+    n, parts = int(rng.integers(2, 10)), int(rng.integers(1, 7))
+    dtype = ("f32", "f16", "bf16")[seed % 3]
+    chunk_elems = int(rng.choice([1, 3, 4, 8, 12, 37, 64, 100, 257]))
+    elems = parts * chunk_elems + int(rng.integers(0, 3))
+    text, table = random_row_list(rng, n, parts, int(rng.integers(1, 11)))
+    main = sarlib.parse(text, n)
+    inputs = make_inputs(n, elems, dtype, seed=seed, kind="ints" if seed % 2 else "normal", scale=2.0)
+    want = [x.copy() for x in inputs]
+    apply_row_list(oracle, table, want, parts, dtype)
+    for t in PLAN_SETTINGS:
+        rows, ptrs = sarlib.plan_rows(main, n, elems * ES[dtype], dtype, executor=1, **t)
+        got = [x.copy() for x in inputs]
+        carry_out_plan(oracle, rows, ptrs, got, dtype)
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "seed %d settings %r rank %d\n%s" % (seed, t, r, text))
+
+
+def test_plan_rows_errors(sarlib):
+    import stragglar_amd as sa
+    S = sarlib.pad_bytes(1 << 20, 8)
+    with pytest.raises(sa.SarError) as ei:
+        sarlib.plan_rows(sarlib.builtin("stragglar", 8), 8, S, executor=0)                    # one launch per round: no column plan
+    assert ei.value.code == -7
+    with pytest.raises(sa.SarError):
+        sarlib.plan_rows(sarlib.builtin("stragglar", 8), 8, S, same_launch=True)              # no pre-work given
+    with pytest.raises(sa.SarError):
+        sarlib.plan_rows(sarlib.builtin("direct", 8), 8, S, prework=sarlib.builtin("prework_ar", 8), same_launch=True)   # chunking differs
