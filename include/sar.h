@@ -131,6 +131,10 @@ typedef struct sar_tuning_t {
                           /*     before a later row overwrites it (partial sums of ring and halving- */
                           /*     doubling, the pre-work's result in a same-launch run) is not stored;*/
                           /*     the buffers after sar_run are the same either way                  */
+    int32_t col_fuse_chains; /* column executor: 1 = a chain of one-sided reduces whose partial sums are  */
+                          /*     neither stored nor read by anyone else (a ring's reduce-scatter)   */
+                          /*     runs as one multi-source row, all its cold operands loaded together */
+                          /*     (in the plan for few work items, where the round trips are the cost) */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

@@ -47,8 +47,17 @@ public:
         choose_shape();
         index_cells();
         Forwarding fwd = choose_forwarding();
+        const Shape before = shape();
+        if (fwd.nslots && env_.tune.col_elide_stores) {
+            mark_dead_stores(fwd);
+            // (in the bandwidth regime the chain is bound by memory either way: measured equal to 2 % slower)
+            if (env_.tune.col_fuse_chains && plan_.staged) fuse_chains(fwd);
+        }
+        if (plan_.staged && env_.tune.col_slots == 0 && fwd.nslots && !slots_pay_when_staged(fwd)) {
+            restore(before);
+            fwd = forward(0); all_found_ = false;
+        }
         plan_.nslots = fwd.nslots; plan_.forwarded_bytes = fwd.bytes;
-        if (fwd.nslots && env_.tune.col_elide_stores) mark_dead_stores(fwd);
         for (uint32_t i = 0; i < nrows(); ++i) { cr_[i].d.flags |= fwd.flags[i]; cr_[i].d.slots = fwd.slots[i]; }
         choose_launch();
         for (const auto& r : cr_) { rows.push_back(r.d); plan_.multi_source |= r.d.kind == SAR_OP_MREDUCE; }
@@ -336,17 +345,105 @@ private:
         uint64_t moved = 0;                  // algorithmic bytes of the rows
         for (const auto& r : cr_) moved += r.d.bytes * (r.d.kind == SAR_OP_COPY ? 2u : r.d.kind == SAR_OP_XREDUCE ? 4u : r.d.kind == SAR_OP_MREDUCE ? r.d.nsrc + r.d.ndst : 3u);
         if (fwd.bytes * 10u < moved) { fwd = forward(0); all_found_ = false; }
-        if (plan_.staged && fwd.nslots) {
-            // Latency plan: the buffers sit in L2 and an operand from there arrives about as fast as one from a
-            // slot.  What forwarding buys is rows that load nothing at all (copies of a held value: no round trip
-            // in the chain).  Keep it when two thirds of the rows are such (the broadcast trees of the StragglAR
-            // tables and of direct: n = 32 at 1 MiB per rank 17.8 us against 21.8 us), not for chains whose
-            // rows mostly still load (ring, halving-doubling: 12.9 against 11.7 us at n = 8).
-            uint32_t free_rows = 0;
-            for (uint32_t i = 0; i < nrows(); ++i) free_rows += cr_[i].d.kind == SAR_OP_COPY && (fwd.flags[i] & DEVOP_GET1);
-            if (free_rows * 3u < nrows() * 2u) { fwd = forward(0); all_found_ = false; }
-        }
         return fwd;
+    }
+
+    // Latency plan: the buffers sit in L2 and an operand from there arrives about as fast as one from a slot.
+    // What forwarding buys is rows that load nothing at all (copies of a held value: no round trip in the
+    // chain).  Keep it when two thirds of the rows are such (the broadcast trees of the StragglAR tables and of
+    // direct: n = 32 at 1 MiB per rank 17.8 us against 21.8 us; ring once its reduce-scatter chain is one row),
+    // not for rows that mostly still load (halving-doubling: 12.9 against 11.7 us at n = 8).
+    bool slots_pay_when_staged(const Forwarding& fwd) const {
+        uint32_t free_rows = 0;
+        for (uint32_t i = 0; i < nrows(); ++i) free_rows += cr_[i].d.kind == SAR_OP_COPY && (fwd.flags[i] & DEVOP_GET1);
+        return free_rows * 3u >= nrows() * 2u;
+    }
+
+    // what fuse_chains changes, to be able to take it back
+    struct Shape {
+        std::vector<ColRow> cr; std::vector<uint32_t> group_begin; std::vector<ColumnComp> comps;
+        uint32_t max_comp_rows, max_comp_groups; size_t nptrs; uint64_t elided;
+    };
+    Shape shape() const { return {cr_, plan_.group_begin, plan_.comps, plan_.max_comp_rows, plan_.max_comp_groups, ptrs_.size(), plan_.elided_bytes}; }
+    void restore(const Shape& sh) {
+        cr_ = sh.cr; plan_.group_begin = sh.group_begin; plan_.comps = sh.comps;
+        plan_.max_comp_rows = sh.max_comp_rows; plan_.max_comp_groups = sh.max_comp_groups;
+        ptrs_.resize(sh.nptrs); plan_.elided_bytes = sh.elided;
+    }
+
+    // Chains of one-sided reduces.  `b += a; c += b; d += c; ...` where every partial sum has the next row as its
+    // only reader, comes to it in a slot and is never stored (the reduce-scatter half of a ring) is one
+    // multi-source row: a + b, then + c, + d in the same order, with all cold operands loaded together instead of
+    // one round trip per row.  It takes the place of the chain's last row; the loads it moves there from earlier
+    // rounds read cells that nobody writes in between (the rows' own stores were dead).
+    void fuse_chains(Forwarding& fwd) {
+        auto plain = [&](uint32_t i) {
+            const DevOp& d = cr_[i].d;
+            return d.kind == SAR_OP_REDUCE_INTO && (d.flags & DEVOP_VEC) && !(d.flags >> DEVOP_HEAD_SHIFT & 15u) && !(d.bytes & 15u) && cr_[i].c0 != cr_[i].c1;
+        };
+        auto written_between = [&](int cell, uint32_t after, uint32_t upto) {      // a row in (after, upto] writes the cell
+            for (auto it = first_after(cell, after); it != ev_[(size_t)cell].end() && it->row <= upto; ++it) if (it->writes) return true;
+            return false;
+        };
+        std::vector<char> removed(nrows(), 0), taken(nrows(), 0);
+        std::vector<std::pair<uint32_t, ColRow>> fused;          // (row replaced, the multi-source row)
+        for (uint32_t i = 0; i < nrows(); ++i) {
+            if (taken[i] || !plain(i) || (fwd.flags[i] & (DEVOP_GET0 | DEVOP_GET1))) continue;
+            std::vector<uint32_t> chain{i};
+            for (uint32_t cur = i;;) {
+                const uint32_t want = DEVOP_PUT | DEVOP_DEAD0;
+                if ((fwd.flags[cur] & want) != want) break;
+                const int cell = cr_[cur].c0;
+                const uint32_t j = next_read(cell, cur);
+                if (j == kNever || taken[j] || !plain(j) || cr_[j].c1 != cell || cr_[j].d.bytes != cr_[cur].d.bytes) break;
+                if ((fwd.flags[j] & (DEVOP_GET0 | DEVOP_GET1)) != DEVOP_GET1 || (fwd.slots[j] >> 8 & 0xffu) != (fwd.slots[cur] >> 16 & 0xffu)) break;
+                if (next_read(cell, j) != kNever) break;                            // somebody else reads the partial sum too
+                chain.push_back(j); cur = j;
+            }
+            if (chain.size() < 2) continue;
+            const uint32_t last = chain.back();
+            bool safe = !written_between(cr_[chain[0]].c1, chain[0], last);
+            for (size_t k = 0; k + 1 < chain.size() && safe; ++k) safe = !written_between(cr_[chain[k]].c0, chain[k], last);
+            if (!safe) continue;
+            ColRow f = cr_[last];
+            f.d.kind = SAR_OP_MREDUCE;
+            f.d.ptr_off = (uint32_t)ptrs_.size(); f.d.nsrc = (uint32_t)chain.size() + 1u; f.d.ndst = 1;
+            ptrs_.push_back(cr_[chain[0]].d.p1); f.mreads.push_back(cr_[chain[0]].c1);
+            for (uint32_t r : chain) { ptrs_.push_back(cr_[r].d.p0); f.mreads.push_back(cr_[r].c0); }
+            ptrs_.push_back(cr_[last].d.p0); f.mwrites.push_back(cr_[last].c0);
+            f.d.p1 = cr_[chain[0]].d.p1; f.c1 = cr_[chain[0]].c1;
+            for (uint32_t r : chain) taken[r] = 1;
+            for (size_t k = 0; k + 1 < chain.size(); ++k) removed[chain[k]] = 1;
+            fused.emplace_back(last, f);
+        }
+        if (fused.empty()) return;
+        for (const auto& fr : fused) {
+            cr_[fr.first] = fr.second;
+            fwd.flags[fr.first] &= DEVOP_PUT | DEVOP_DEAD0; fwd.slots[fr.first] &= 0xff0000u;
+        }
+        // take the fused-away rows out: same components, groups that became empty disappear
+        std::vector<ColRow> cr; std::vector<uint32_t> flags, slots, group_begin; std::vector<ColumnComp> comps;
+        uint32_t max_rows = 0, max_groups = 0;
+        for (const auto& cc : plan_.comps) {
+            ColumnComp nc{};
+            nc.group_first = (uint32_t)group_begin.size(); nc.row_first = (uint32_t)cr.size();
+            for (uint32_t g = cc.group_first; g < cc.group_end; ++g) {
+                bool open = false;
+                for (uint32_t i = plan_.group_begin[g]; i < plan_.group_begin[g + 1]; ++i) {
+                    if (removed[i]) continue;
+                    if (!open) { group_begin.push_back((uint32_t)cr.size()); open = true; }
+                    cr.push_back(cr_[i]); flags.push_back(fwd.flags[i]); slots.push_back(fwd.slots[i]);
+                }
+            }
+            nc.group_end = (uint32_t)group_begin.size(); nc.row_end = (uint32_t)cr.size();
+            max_rows = std::max(max_rows, nc.row_end - nc.row_first); max_groups = std::max(max_groups, nc.group_end - nc.group_first);
+            comps.push_back(nc);
+        }
+        group_begin.push_back((uint32_t)cr.size());
+        cr_.swap(cr); fwd.flags.swap(flags); fwd.slots.swap(slots);
+        plan_.group_begin.swap(group_begin); plan_.comps.swap(comps);
+        plan_.max_comp_rows = max_rows; plan_.max_comp_groups = max_groups;
+        ev_.clear();                            // row numbers have changed
     }
 
     // Stores nobody needs.  A row's result for a cell is dead when a later row overwrites the cell and every row

@@ -64,7 +64,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -459,7 +459,7 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
-           (t.col_elide_stores == 0 || t.col_elide_stores == 1);
+           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1);
 }
 
 // sar_plan / sar_plan_rows: a context that never touches the device, with the rank buffers at made-up, suitably

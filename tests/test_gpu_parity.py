@@ -218,7 +218,8 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
                   dict(col_forward=1, col_latency_plan=1), dict(col_forward=1, col_latency_plan=2, col_slots=2),
                   dict(col_forward=0, col_latency_plan=2, cache_policy=1),
                   dict(col_forward=1, col_split=0), dict(col_forward=0, col_split=0), dict(col_forward=1, col_split=0, col_latency_plan=2),
-                  dict(col_forward=1, col_elide_stores=0), dict(col_forward=1, col_elide_stores=0, col_slots=2, col_latency_plan=2)):
+                  dict(col_forward=1, col_elide_stores=0), dict(col_forward=1, col_elide_stores=0, col_slots=2, col_latency_plan=2),
+                  dict(col_forward=1, col_fuse_chains=0, col_slots=2, col_latency_plan=2), dict(col_forward=1, col_slots=1, col_latency_plan=2, col_wgs=1)):
             # these buffers have few columns: unless a case asks for it, keep the plan for few work items out of the way
             got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(dict(col_latency_plan=0), **dict(t, executor=1)))
             st = gpu_ctx.stats()

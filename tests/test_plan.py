@@ -89,9 +89,21 @@ def test_small_messages_take_the_plan_for_few_items(sarlib):
     st = plan(sarlib, "stragglar", 8, S)
     assert st.executor == 1 and st.launches == 1 and st.col_block == 256 and st.col_components == 7
     assert st.col_slots == 1                                  # broadcast trees keep forwarding there
+    rhd = plan(sarlib, "rhd", 8, S)
+    assert rhd.executor == 1 and rhd.col_slots == 0           # rows that mostly still load do not
+    assert plan(sarlib, "rhd", 8, S, col_latency_plan=0).col_slots == 4
+    # ring: the reduce-scatter chain of a chunk becomes one multi-source row, and what is left are copies of its result
     ring = plan(sarlib, "ring", 8, S)
-    assert ring.executor == 1 and ring.col_slots == 0         # chains whose rows mostly still load do not
-    assert plan(sarlib, "ring", 8, S, col_latency_plan=0).col_slots == 1
+    assert ring.executor == 1 and ring.col_slots == 1
+    assert plan(sarlib, "ring", 8, S, col_fuse_chains=0).col_slots == 0
+    rows, ptrs = sarlib.plan_rows(sarlib.builtin("ring", 8), 8, S)
+    assert [r.kind for r in rows if r.component == 0] == [3] + [0] * 7
+    first = rows[0]
+    assert (first.nsrc, first.ndst, first.put_slot, first.dead0) == (8, 1, 0, 0)
+    # allreduce_8GPU.cu:154-193: chunk c is summed along the ring c+1, c+2, ..., c; rank c's copy is the result
+    chunk = S // 8
+    c = ptrs[first.first_ptr][1] // chunk
+    assert [rank for rank, _ in ptrs[first.first_ptr:first.first_ptr + 9]] == [(c + 1 + k) % 8 for k in range(8)] + [c]
 
 
 def test_prework_and_misaligned_buffers(sarlib):
