@@ -130,6 +130,31 @@ def test_larger_rank_counts(gpu_ctx, sarlib, oracle, n, table):
                 assert_bits_equal(g[r], w[r], "%s n=16 rank %d" % (alg, r))
 
 
+@pytest.mark.parametrize("n", [48, 64])
+def test_most_ranks_the_library_takes(gpu_ctx, sarlib, oracle, n):
+    """Up to SAR_MAX_RANKS = 64 emulated ranks, tables from this package's own synthesizers (the reference ships
+    none beyond 8; simulation.py:7 goes to 192).  Whatever valid table is used, every rank must end with the
+    pre-work's ring-ordered sum plus the straggler's value: the checker runs the same table."""
+    from stragglar_amd import _synth, synthesizer_nonpow2, synthesizer_pow2
+    text = _synth.table_text((synthesizer_pow2 if n & (n - 1) == 0 else synthesizer_nonpow2).construct_schedule(n))
+    elems = (n - 1) * 260 + 5
+    for dtype in ("f32", "bf16"):
+        inputs = make_inputs(n, elems, dtype, seed=n, kind="ints")
+        want = run_oracle(oracle, "stragglar", inputs, dtype, text, delay=0.0)
+        total = np.sum([from_bits(x, dtype) for x in inputs], axis=0)
+        assert np.array_equal(from_bits(want[0], dtype)[:(n - 1) * 260], total[:(n - 1) * 260])      # small integers: exact in any order
+        for t in (dict(), dict(executor=0), dict(executor=1, col_latency_plan=0), dict(executor=1, col_split=0, col_slots=6)):
+            got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, text, delay=0.0, tuning=t)
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "n=%d %s tuning %r rank %d" % (n, dtype, t, r))
+    for alg in ("ring", "direct") + (("rhd",) if n == 64 else ()):
+        inputs = make_inputs(n, n * 64 + 3, "f32", seed=n + 1)
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, "f32", None, delay=0.0)
+        want = run_oracle(oracle, alg, inputs, "f32", None, delay=0.0)
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s n=%d rank %d" % (alg, n, r))
+
+
 @pytest.mark.parametrize("executor", [0, 1, 2])
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 8 * 7 * 4 * 13 + 5, 7 * 8 * 2051])
