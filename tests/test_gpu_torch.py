@@ -111,3 +111,39 @@ def test_adopt_rejects_bad_buffers(sarlib):
         assert torch.all(t[:512] == 2.0) and torch.all(t[512:] == 3.0)
     finally:
         ctx.close()
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.float32, "f32"), (torch.bfloat16, "bf16")])
+@pytest.mark.parametrize("shifts", ["same", "mixed"])
+def test_rank_tensors_that_start_off_the_vector_boundary(oracle, dtype, name, shifts):
+    """Views into a larger allocation, as a caller's flat gradient slices would be: every rank tensor starts a few
+    elements past a 16-byte boundary.  With the same distance in all ranks the rows still run as vectors (moved up
+    to the boundary, the bytes in front element by element); with different distances they run element by element.
+    Either way the bits are the checker's."""
+    from stragglar_amd.torch_emulation import EmulatedGroup
+    n, numel = 8, 7 * 8 * 515
+    for alg in ("stragglar", "ring", "rhd", "direct"):
+        g = torch.Generator(device="cpu").manual_seed(11)
+        pool = torch.zeros(n * (numel + 64), dtype=dtype, device="cuda")
+        tensors = []
+        for r in range(n):
+            shift = 3 if shifts == "same" else (1, 3, 0, 5, 2, 7, 4, 6)[r]
+            v = pool[r * (numel + 64) + shift:r * (numel + 64) + shift + numel]
+            v.copy_((torch.rand(numel, generator=g, dtype=torch.float32) * 2 - 1).to(dtype))
+            tensors.append(v)
+        assert all(t.data_ptr() % 16 for t in tensors if shifts == "same")
+        inputs = [to_np_bits(t).copy() for t in tensors]
+        group = EmulatedGroup(n, algorithm=alg)
+        try:
+            group.all_reduce(tensors)
+            want = [x.copy() for x in inputs]
+            oracle.run(alg, want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")) if alg == "stragglar" else None, delay=0.0)
+            for r in range(n):
+                assert_bits_equal(to_np_bits(tensors[r]), want[r], "%s %s shifts, rank %d" % (alg, shifts, r))
+            # nothing outside the views was touched
+            for r in range(n):
+                lo, hi = r * (numel + 64), (r + 1) * (numel + 64)
+                shift = 3 if shifts == "same" else (1, 3, 0, 5, 2, 7, 4, 6)[r]
+                assert torch.all(pool[lo:lo + shift] == 0) and torch.all(pool[lo + shift + numel:hi] == 0)
+        finally:
+            group.close()
