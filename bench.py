@@ -198,6 +198,8 @@ def main():
         "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),
         "wall_ms_per_step_back_to_back": round(back_to_back_ms, 4),
         "ranks_identical_after_run": bool(identical),
+        # 1 = the two halves of the rank buffers were placed in different regions of HBM (sar_alloc_ranks)
+        "arena_spread": int(st.arena_spread),
         "roofline": roofline,
     }
     if st.col_slots and args.forward is None:

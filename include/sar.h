@@ -82,7 +82,7 @@ typedef struct sar_stats_t {
     uint64_t forwarded_bytes;      /* part of algorithmic_bytes that the column executor takes from value slots   */
                                    /* in LDS instead of loading it again from the rank buffers                    */
     int32_t fused_prework;         /* 1 if sar_run(delay 0) runs pre-work + main schedule as a single launch      */
-    int32_t reserved;
+    int32_t arena_spread;          /* 1 if the two halves of the rank buffers lie in different regions of HBM    */
     uint64_t elided_store_bytes;   /* part of algorithmic_bytes that the column executor does not store because a */
                                    /* later row overwrites it and every reader in between takes it from a slot    */
 } sar_stats_t;
@@ -135,6 +135,12 @@ typedef struct sar_tuning_t {
                           /*     neither stored nor read by anyone else (a ring's reduce-scatter)   */
                           /*     runs as one multi-source row, all its cold operands loaded together */
                           /*     (in the plan for few work items, where the round trips are the cost) */
+    int32_t arena_spread; /* sar_alloc_ranks: 1 = for payloads of 128 MiB and more, half the ranks go   */
+                          /*     into an allocation of their own that a short timing probe has shown */
+                          /*     to lie in another region of HBM than the first half's (MI355X:     */
+                          /*     buffers in different thirds of the 288 GiB disturb each other less; */
+                          /*     the pair is kept for the life of the context); ranks back to back  */
+                          /*     when no such pair is found or the device lacks the room; 0 = never  */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

@@ -41,7 +41,7 @@ class Stats(ctypes.Structure):
                 ("prework_bytes", ctypes.c_uint64), ("rounds", ctypes.c_int32), ("launches", ctypes.c_int32),
                 ("ops", ctypes.c_int32), ("uses_graph", ctypes.c_int32), ("executor", ctypes.c_int32),
                 ("col_block", ctypes.c_int32), ("col_slots", ctypes.c_int32), ("col_components", ctypes.c_int32),
-                ("forwarded_bytes", ctypes.c_uint64), ("fused_prework", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("forwarded_bytes", ctypes.c_uint64), ("fused_prework", ctypes.c_int32), ("arena_spread", ctypes.c_int32),
                 ("elided_store_bytes", ctypes.c_uint64)]
 
 
@@ -60,7 +60,7 @@ class PlanPtr(ctypes.Structure):
 
 class Tuning(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd", "segments",
-                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains")]
+                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "arena_spread")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

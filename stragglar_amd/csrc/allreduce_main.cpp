@@ -204,9 +204,9 @@ int main(int argc, char* argv[]) {
         double mean = sum_ms / numIters;
         fprintf(stderr, "# algorithmic_bytes=%.0f mean_ms=%.4f min_ms=%.4f algorithmic_GBps=%.1f (best %.1f) hbm_roofline_frac=%.3f launches=%d graph=%d\n",
                 total, mean, min_ms, total / mean / 1e6, total / min_ms / 1e6, total / mean / 1e6 / 8000.0, st.launches, st.uses_graph);
-        fprintf(stderr, "# executor=%s components=%d column_threads=%d value_slots=%d forwarded_bytes=%.0f elided_store_bytes=%.0f memory_side_GBps=%.1f prework_in_same_launch=%d\n",
+        fprintf(stderr, "# executor=%s components=%d column_threads=%d value_slots=%d forwarded_bytes=%.0f elided_store_bytes=%.0f memory_side_GBps=%.1f prework_in_same_launch=%d ranks_in_two_hbm_regions=%d\n",
                 st.executor ? "column" : "rounds", st.col_components, st.col_block, st.col_slots, (double)st.forwarded_bytes, (double)st.elided_store_bytes,
-                (total - (double)st.forwarded_bytes - (double)st.elided_store_bytes) / mean / 1e6, (sleepTime == 0 && st.fused_prework) ? 1 : 0);
+                (total - (double)st.forwarded_bytes - (double)st.elided_store_bytes) / mean / 1e6, (sleepTime == 0 && st.fused_prework) ? 1 : 0, st.arena_spread);
     }
 
     // result check (allreduce_8GPU.cu:1069-1077 asserts 36.0; allreduce_4GPU.cu:593-603 prints mismatches)

@@ -29,6 +29,11 @@ int set_error(int code, const std::string& msg) { g_error = msg; return code; }
     } while (0)
 
 constexpr uint64_t kArenaAlign = 2ull << 20;   // rank bases on 2 MiB boundaries (one large-page fragment each)
+constexpr uint64_t kSpreadMinPayload = 128ull << 20;   // spread arena: from 16 MiB per rank at n = 8 (below, the caches carry the schedule)
+constexpr uint64_t kSpreadHeadroom = 16ull << 30;      // memory left alone while looking for the pair
+constexpr uint64_t kSpreadMinAlloc = 8ull << 30, kSpreadMaxAlloc = 32ull << 30;      // per half; one size serves most payloads
+constexpr uint64_t kSpreadSearch = 112ull << 30;       // candidates held while looking: a region and a bit
+constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 streams of this size (beyond what the Infinity Cache absorbs)
 constexpr float kMaxDelayMs = 60000.f;
 
 // One kernel launch: the rows of a round that share a kernel (COPY /
@@ -60,11 +65,17 @@ struct sar_ctx {
 
     int n = 0, dtype = SAR_F32;
     uint64_t bytes_per_rank = 0, stride = 0;
-    char* arena = nullptr;
+    char* arena = nullptr;             // ranks [0, split) at arena + r * stride
+    char* arena_hi = nullptr;          // ranks [split, n) at arena_hi + (r - split) * stride (spread arena only)
+    int split = 0;
+    char* pair_lo = nullptr;           // the spread arena's two allocations, pair_bytes each, found to lie in
+    char* pair_hi = nullptr;           // different regions of HBM; kept for the life of the context
+    uint64_t pair_bytes = 0;
+    bool spread_capable = false;       // the device is one whose regions are known (MI355X, 288 GiB)
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -84,7 +95,11 @@ struct sar_ctx {
     std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
 
     bool has_ranks() const { return arena != nullptr || !adopted.empty(); }
-    char* rank_base(int r) const { return adopted.empty() ? arena + (uint64_t)r * stride : adopted[(size_t)r]; }
+    char* rank_base(int r) const {
+        if (!adopted.empty()) return adopted[(size_t)r];
+        return r < split ? arena + (uint64_t)r * stride : arena_hi + (uint64_t)(r - split) * stride;
+    }
+    bool spread() const { return adopted.empty() && arena != nullptr && split < n; }
     uint64_t elems() const { return bytes_per_rank / (uint64_t)elem_size_of(dtype); }
     uint64_t snapshot_stride() const { return adopted.empty() ? stride : (bytes_per_rank + 255u) & ~(uint64_t)255u; }
 };
@@ -106,9 +121,75 @@ void drop_plan(sar_ctx* c) {
     c->stats = sar_stats_t{};
 }
 
+void drop_pair(sar_ctx* c) {
+    if (c->pair_lo) (void)hipFree(c->pair_lo);
+    if (c->pair_hi) (void)hipFree(c->pair_hi);
+    c->pair_lo = c->pair_hi = nullptr; c->pair_bytes = 0;
+}
+
+// Best of `reps` runs of the region probe on two windows of 4 * kProbeStream bytes, in milliseconds as the kernel
+// timed itself on the device's wall clock; negative on error.
+float probe_ms(sar_ctx* c, char* a, char* b, int reps) {
+    unsigned long long* stamps = nullptr;
+    if (hipMalloc((void**)&stamps, 2 * sizeof(unsigned long long)) != hipSuccess) { (void)hipGetLastError(); return -1.f; }
+    float best = -1.f;
+    for (int i = 0; i < reps; ++i) {
+        unsigned long long h[2] = {~0ull, 0ull};
+        if (hipMemcpyAsync(stamps, h, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+            sar::launch_region_probe(c->stream, a, b, kProbeStream, stamps) != hipSuccess ||
+            hipMemcpyAsync(h, stamps, sizeof(h), hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+            hipStreamSynchronize(c->stream) != hipSuccess || h[1] <= h[0]) { (void)hipGetLastError(); best = -1.f; break; }
+        const float ms = (float)((double)(h[1] - h[0]) / (double)c->wall_khz);
+        if (best < 0.f || ms < best) best = ms;
+    }
+    (void)hipFree(stamps);
+    return best;
+}
+
+// Two allocations of `bytes` each that lie in different regions of HBM.  Measured on MI355X: the 288 GiB behave as
+// three regions of 96 GiB (presumably the stack levels of the 12-high HBM3E), and streams that run at the same
+// time in different regions get in each other's way less: the write-heavy schedules here gain 15 to 25 %, and
+// which region a buffer falls in is all that matters, not where in it.  Where an allocation lands physically is
+// the driver's business, so candidates are allocated one after the other and each is timed against the first
+// with a short probe (eight write streams of 128 MiB, four in either allocation: 182-212 us when both lie in
+// the same region, 156-162 us when they do not, on every box seen) until one turns out to lie elsewhere; the
+// others are given back.  Nothing is assumed about the order in which the driver hands out memory, and a wrong
+// verdict costs speed, not correctness: without a pair the caller falls back to one allocation.
+bool find_spread_pair(sar_ctx* c, uint64_t bytes) {
+    const uint64_t window = 4 * kProbeStream;
+    const float elsewhere_ms = (float)(8.0 * (double)kProbeStream / 6.3e9);      // the probe's 1 GiB at 6.3 TB/s: 170 us
+    if (bytes < 2 * window) return false;
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); return false; }
+    if (free_b < 4 * bytes + kSpreadHeadroom) return false;
+    // enough candidates to cross a region boundary from anywhere, no more
+    const uint64_t budget = std::min<uint64_t>((uint64_t)free_b - kSpreadHeadroom, kSpreadSearch + 2 * bytes);
+    char* lo = nullptr;
+    if (hipMalloc((void**)&lo, bytes) != hipSuccess) { (void)hipGetLastError(); return false; }
+    std::vector<char*> held;
+    char* hi = nullptr;
+    for (uint64_t used = bytes; used + bytes <= budget; used += bytes) {
+        char* cand = nullptr;
+        if (hipMalloc((void**)&cand, bytes) != hipSuccess) { (void)hipGetLastError(); break; }
+        const float t = probe_ms(c, lo, cand, 3);
+        if (t < 0.f) { (void)hipFree(cand); break; }
+        // elsewhere if fast twice, on different windows of both
+        if (t < elsewhere_ms) {
+            const float t2 = probe_ms(c, lo + bytes - window, cand + bytes - window, 3);
+            if (t2 > 0.f && t2 < elsewhere_ms) { hi = cand; break; }
+        }
+        held.push_back(cand);
+    }
+    for (char* p : held) (void)hipFree(p);
+    if (!hi) { (void)hipFree(lo); return false; }
+    c->pair_lo = lo; c->pair_hi = hi; c->pair_bytes = bytes;
+    return true;
+}
+
 void drop_ranks(sar_ctx* c) {
     drop_plan(c);
-    if (c->arena) { (void)hipFree(c->arena); c->arena = nullptr; }
+    if (c->arena && c->arena != c->pair_lo) (void)hipFree(c->arena);
+    c->arena = c->arena_hi = nullptr; c->split = 0;
     if (c->snapshot) { (void)hipFree(c->snapshot); c->snapshot = nullptr; }
     c->adopted.clear();
     c->n = 0; c->bytes_per_rank = 0; c->stride = 0;
@@ -447,6 +528,7 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     st.forwarded_bytes = column ? cp.forwarded_bytes : 0;
     st.elided_store_bytes = column ? cp.elided_bytes : 0;
     st.fused_prework = fused ? 1 : 0;
+    st.arena_spread = c->spread() ? 1 : 0;
     return st;
 }
 
@@ -459,7 +541,8 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
-           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1);
+           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1) &&
+           (t.arena_spread == 0 || t.arena_spread == 1);
 }
 
 // sar_plan / sar_plan_rows: a context that never touches the device, with the rank buffers at made-up, suitably
@@ -593,6 +676,12 @@ int sar_create(int device, sar_ctx** out) {
     }
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0) c->cu_count = cus;
+    {
+        // three regions of 96 GiB (see find_spread_pair); only known for the 288 GiB of MI355X
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) == hipSuccess && total_b >= (280ull << 30) && total_b <= (290ull << 30)) c->spread_capable = true;
+        else (void)hipGetLastError();
+    }
     int khz = 0;
     if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0) c->wall_khz = khz;
     *out = c;
@@ -605,6 +694,7 @@ void sar_destroy(sar_ctx* c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     if (c->straggler_stream) (void)hipStreamSynchronize(c->straggler_stream);
     drop_ranks(c);
+    drop_pair(c);
     for (auto e : c->ev_prof) (void)hipEventDestroy(e);
     if (c->d_flag) (void)hipFree(c->d_flag);
     if (c->ev_start) (void)hipEventDestroy(c->ev_start);
@@ -624,8 +714,28 @@ int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_ranks(c);
     uint64_t stride = (bytes_per_rank + kArenaAlign - 1) / kArenaAlign * kArenaAlign;
-    hipError_t e = hipMalloc((void**)&c->arena, stride * (uint64_t)n);
-    if (e != hipSuccess) { (void)hipGetLastError(); c->arena = nullptr; return set_error(SAR_ENOMEM, std::string("rank arena: ") + hipGetErrorString(e)); }
+    // Spread arena: half the ranks in an allocation of their own that lies in another region of HBM than the
+    // first half's (find_spread_pair).  Only for payloads that are bound by memory, and only when the device has
+    // the room to look for such a pair; otherwise the ranks sit back to back.
+    const int half = (n + 1) / 2;
+    const uint64_t payload = stride * (uint64_t)n;
+    bool spread = c->tune.arena_spread != 0 && c->spread_capable && payload >= kSpreadMinPayload;
+    if (spread) {
+        uint64_t need = kSpreadMinAlloc;
+        while (need < stride * (uint64_t)half) need <<= 1;
+        if (c->pair_bytes < need) { drop_pair(c); spread = need <= kSpreadMaxAlloc && find_spread_pair(c, need); }
+    }
+    if (spread) {
+        c->arena = c->pair_lo; c->arena_hi = c->pair_hi; c->split = half;
+    } else {
+        hipError_t e = hipMalloc((void**)&c->arena, payload);
+        if (e != hipSuccess && c->pair_lo) {       // the idle spread arena may be what is in the way
+            (void)hipGetLastError(); drop_pair(c);
+            e = hipMalloc((void**)&c->arena, payload);
+        }
+        if (e != hipSuccess) { (void)hipGetLastError(); c->arena = nullptr; return set_error(SAR_ENOMEM, std::string("rank arena: ") + hipGetErrorString(e)); }
+        c->arena_hi = nullptr; c->split = n;
+    }
     c->n = n; c->dtype = dtype; c->bytes_per_rank = bytes_per_rank; c->stride = stride;
     return SAR_OK;
 }
@@ -733,7 +843,7 @@ int sar_snapshot(sar_ctx* c) {
         hipError_t e = hipMalloc((void**)&c->snapshot, stride * (uint64_t)c->n);
         if (e != hipSuccess) { (void)hipGetLastError(); c->snapshot = nullptr; return set_error(SAR_ENOMEM, std::string("snapshot: ") + hipGetErrorString(e)); }
     }
-    if (c->adopted.empty()) {
+    if (c->adopted.empty() && !c->spread()) {
         SAR_HIP(hipMemcpyAsync(c->snapshot, c->arena, stride * (uint64_t)c->n, hipMemcpyDeviceToDevice, c->stream));
     } else {
         for (int r = 0; r < c->n; ++r)
@@ -747,7 +857,7 @@ int sar_restore(sar_ctx* c) {
     if (!c || !c->has_ranks() || !c->snapshot) return set_error(SAR_ESTATE, "no snapshot taken");
     SAR_HIP(hipSetDevice(c->device));
     const uint64_t stride = c->snapshot_stride();
-    if (c->adopted.empty()) {
+    if (c->adopted.empty() && !c->spread()) {
         SAR_HIP(hipMemcpyAsync(c->arena, c->snapshot, stride * (uint64_t)c->n, hipMemcpyDeviceToDevice, c->stream));
     } else {
         for (int r = 0; r < c->n; ++r)

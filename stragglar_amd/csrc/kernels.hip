@@ -674,6 +674,30 @@ hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t
     hipLaunchKernelGGL(compare_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, a, b, bytes, differs);
     return hipGetLastError();
 }
+// Region probe: four write streams in window a and four in window b, stream_bytes each, all running at once.
+// How long it takes tells whether the two windows lie in the same region of HBM (see find_spread_pair in
+// executor.cpp).  The kernel times itself on the device's constant-rate wall clock -- stamps[0] = earliest start,
+// stamps[1] = latest end with all stores acknowledged, preset by the host to ~0 and 0 -- so that neither launch
+// overhead nor a profiler's bookkeeping enters the figure.
+__global__ __launch_bounds__(256) void region_probe_kernel(char* a, char* b, uint64_t stream_bytes, unsigned long long* stamps) {
+    if (threadIdx.x == 0) atomicMin(&stamps[0], (unsigned long long)wall_clock64());
+    const uint64_t nvec = stream_bytes >> 4, step = (uint64_t)gridDim.x * blockDim.x;
+    const f4 v = {1.f, 2.f, 3.f, 4.f};
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += step) {
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; ++k) {
+            st16<false>(a + k * stream_bytes + (i << 4), v);
+            st16<false>(b + k * stream_bytes + (i << 4), v);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");       // this wave's stores acknowledged (no cache write-back)
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(&stamps[1], (unsigned long long)wall_clock64());
+}
+hipError_t launch_region_probe(hipStream_t st, char* a, char* b, uint64_t stream_bytes, unsigned long long* stamps) {
+    hipLaunchKernelGGL(region_probe_kernel, dim3(2048), dim3(256), 0, st, a, b, stream_bytes, stamps);
+    return hipGetLastError();
+}
 hipError_t launch_sleep(hipStream_t st, uint64_t ticks) {
     hipLaunchKernelGGL(sleep_kernel, dim3(1), dim3(1), 0, st, ticks);
     return hipGetLastError();

@@ -83,6 +83,9 @@ hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, h
 hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype);
 hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype);
 hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t bytes, int* differs);
+// writes 4 * stream_bytes to each of the two windows; stamps[0] / stamps[1] (preset to ~0 / 0) receive the wall-clock
+// ticks of the earliest start and the latest end
+hipError_t launch_region_probe(hipStream_t st, char* a, char* b, uint64_t stream_bytes, unsigned long long* stamps);
 hipError_t launch_sleep(hipStream_t st, uint64_t ticks);
 
 }  // namespace sar

@@ -639,3 +639,34 @@ def test_random_row_lists(gpu_ctx, sarlib, oracle, seed):
         ctx.run(-1.0)
         for r in range(n):
             assert_bits_equal(ctx.download(r), want[r], "seed %d n=%d parts=%d chunk %d %s tuning %r rank %d\n%s" % (seed, n, parts, chunk_elems, dtype, t, r, text))
+
+
+def test_spread_arena(gpu_ctx, sarlib, oracle):
+    """From 128 MiB of payload sar_alloc_ranks puts half the ranks 96 GiB above the others (one allocation; MI355X's
+    HBM behaves as three regions of 96 GiB and buffers in different regions disturb each other less).  Where the
+    ranks sit must not change a bit, uploads, downloads, fills, snapshots and comparisons included."""
+    n, dtype = 8, "f32"
+    elems = 7 * 8 * 75000 + 5                       # 16.8 MB per rank: 134 MB of payload
+    inputs = make_inputs(n, elems, dtype, seed=77)
+    want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+    seen = []
+    for spread in (1, 0, 1):
+        for executor in (1, 0):
+            gpu_ctx.set_tuning(arena_spread=spread)                 # read when the ranks are allocated
+            got = run_gpu(gpu_ctx, sarlib, "stragglar", n, inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0,
+                          tuning=dict(arena_spread=spread, executor=executor))
+            seen.append(gpu_ctx.stats().arena_spread)
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "spread %d executor %d rank %d" % (spread, executor, r))
+        gpu_ctx.snapshot()
+        gpu_ctx.fill_const(3, 1.0)
+        assert not gpu_ctx.ranks_identical((elems // 7) * 7)
+        gpu_ctx.restore()
+        assert gpu_ctx.ranks_identical((elems // 7) * 7)
+        assert_bits_equal(gpu_ctx.download(5), want[5], "after restore")
+    assert seen[2:4] == [0, 0] and seen[0] == seen[1] == seen[4] == seen[5]      # 1 where the device has the room
+    # small payloads stay back to back
+    small = make_inputs(n, 7 * 8 * 100, dtype, seed=78)
+    gpu_ctx.set_tuning(arena_spread=1)
+    run_gpu(gpu_ctx, sarlib, "stragglar", n, small, dtype, read_golden("stragglar_n8_cu.txt"), tuning=dict(arena_spread=1))
+    assert gpu_ctx.stats().arena_spread == 0
