@@ -216,6 +216,11 @@ def main():
         rec["every_operand_loaded"] = {"value": round(st.algorithmic_bytes / pm / 1e6, 1), "unit": "GB/s", "ms_per_step": round(pm, 5),
                                        "frac_of_hbm_peak": round(st.algorithmic_bytes / pm / 1e6 / HBM_PEAK_GBPS, 4),
                                        "ranks_identical_after_run": bool(ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts))}
+        plain_key = "%s_n%d_%dMiB_f32_column" % (args.alg, n, args.mib)
+        if os.path.exists(tpath) and plain_key in t:
+            # what the counters saw of it: re-reads of an item that hit the XCD's own L2 never reach the fabric
+            rec["every_operand_loaded"]["traffic"] = t[plain_key]["hbm_bytes_per_launch"]
+            rec["every_operand_loaded"]["memory_side_GBps"] = round(t[plain_key]["hbm_bytes_per_launch"] / pm / 1e6, 1)
         ctx.set_tuning(col_forward=1)
         ctx.prepare(main_sched, None, use_graph=False)
     if not args.no_cpu and args.alg == "stragglar":
