@@ -169,7 +169,7 @@ def test_byte_accounting(sarlib):
 
 
 def test_pad_bytes_matches_pad_buffers_py(sarlib):
-    """pad_buffers.py:31-48 and the sizes the survey derived from it."""
+    """pad_buffers.py:31-48 and the padded sizes that follow from it for the benchmark configurations."""
     assert [sarlib.pad_bytes(b, 8) for b in (4096, 65536, 1 << 20, 16 << 20, 256 << 20, 1 << 30)] == \
         [7168, 71680, 1053696, 16780288, 268441600, 1073744896]
     assert sarlib.pad_bytes(1 << 20, 4) == 1050624
