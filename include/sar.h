@@ -135,6 +135,10 @@ typedef struct sar_tuning_t {
                           /*     neither stored nor read by anyone else (a ring's reduce-scatter)   */
                           /*     runs as one multi-source row, all its cold operands loaded together */
                           /*     (in the plan for few work items, where the round trips are the cost) */
+    int32_t col_fuse_copies; /* column executor: 1 = copies of a value that an earlier row of the work   */
+                          /*     item still holds are issued by that row as extra stores, and the    */
+                          /*     copy rows (with their round boundaries) go away, in the plan for    */
+                          /*     few work items; 2 = in every plan; 0 = never                       */
     int32_t arena_spread; /* sar_alloc_ranks: 1 = for payloads of 128 MiB and more, half the ranks go   */
                           /*     into an allocation of their own that a short timing probe has shown */
                           /*     to lie in another region of HBM than the first half's (MI355X:     */
@@ -318,7 +322,8 @@ typedef struct sar_plan_row {
     int32_t dead1;       /* the same for p1 (XREDUCE)                                                           */
     int32_t nsrc;        /* MREDUCE: sources, in add order ...                                                  */
     int32_t ndst;        /* ... and destinations: entries [first_ptr, first_ptr + nsrc + ndst) of the pointer   */
-    int32_t first_ptr;   /* list                                                                                */
+    int32_t first_ptr;   /* list.  Other kinds: nsrc = 0 and ndst further destinations of the result (copies    */
+                         /* of it that later rows would have made), entries [first_ptr, first_ptr + ndst)       */
     int32_t reserved;
 } sar_plan_row;
 

@@ -19,7 +19,7 @@ struct ColRow {
     DevOp d;
     int c0, c1;                        // cells of p0 and p1
     uint32_t round;
-    std::vector<int> mreads, mwrites;  // cells of a multi-source row
+    std::vector<int> mreads, mwrites;  // cells of a multi-source row; mwrites of any other row: its extra destinations
 };
 
 struct Ev { uint32_t row; bool reads, writes; };   // a row touching a cell; a reducing row reads and writes its cell
@@ -53,7 +53,12 @@ public:
             // (in the bandwidth regime the chain is bound by memory either way: measured equal to 2 % slower)
             if (env_.tune.col_fuse_chains && plan_.staged) fuse_chains(fwd);
         }
-        if (plan_.staged && env_.tune.col_slots == 0 && fwd.nslots && !slots_pay_when_staged(fwd)) {
+        const bool pays = !plan_.staged || env_.tune.col_slots != 0 || !fwd.nslots || slots_pay_when_staged(fwd);
+        const uint32_t rows_before = (uint32_t)before.cr.size();
+        if (fwd.nslots && (env_.tune.col_fuse_copies == 2 || (env_.tune.col_fuse_copies == 1 && plan_.staged))) fuse_copies(fwd);
+        // (latency plan) ... or when taking the copies of held values into the rows that produce them shortens the
+        // items by a quarter or more (halving-doubling: the doubling half disappears, 11.4 -> 10.2 us at n = 8)
+        if (!pays && nrows() * 4u > rows_before * 3u) {
             restore(before);
             fwd = forward(0); all_found_ = false;
         }
@@ -228,6 +233,7 @@ private:
             const bool reduce = r.d.kind != SAR_OP_COPY, both = r.d.kind == SAR_OP_XREDUCE;
             ev_[(size_t)r.c0].push_back({i, reduce, true});
             if (r.c1 != r.c0) ev_[(size_t)r.c1].push_back({i, true, both});
+            for (int cell : r.mwrites) ev_[(size_t)cell].push_back({i, false, true});
         }
     }
     std::vector<Ev>::const_iterator first_after(int cell, uint32_t i) const {
@@ -421,7 +427,11 @@ private:
             cr_[fr.first] = fr.second;
             fwd.flags[fr.first] &= DEVOP_PUT | DEVOP_DEAD0; fwd.slots[fr.first] &= 0xff0000u;
         }
-        // take the fused-away rows out: same components, groups that became empty disappear
+        remove_rows(removed, fwd);
+    }
+
+    // Takes rows out of the plan: same components, groups that became empty disappear; the cell index is rebuilt.
+    void remove_rows(const std::vector<char>& removed, Forwarding& fwd) {
         std::vector<ColRow> cr; std::vector<uint32_t> flags, slots, group_begin; std::vector<ColumnComp> comps;
         uint32_t max_rows = 0, max_groups = 0;
         for (const auto& cc : plan_.comps) {
@@ -443,7 +453,52 @@ private:
         cr_.swap(cr); fwd.flags.swap(flags); fwd.slots.swap(slots);
         plan_.group_begin.swap(group_begin); plan_.comps.swap(comps);
         plan_.max_comp_rows = max_rows; plan_.max_comp_groups = max_groups;
-        ev_.clear();                            // row numbers have changed
+        index_cells();                          // row numbers have changed
+    }
+
+    // Copies of a held value.  A row that keeps its result in a slot is often followed, rounds later, by copies of
+    // that very value to other ranks (the broadcast tree of a StragglAR exchange, a ring's all-gather): rows that
+    // load nothing and store one vector.  When nobody touches a copy's destination between the producing row and
+    // the copy, the store can just as well be issued by the producing row: the copy row goes away (with its round
+    // boundary, when it was alone in it) and the producing row gets one more destination.  Only for plans made of
+    // whole vectors; a copy whose store was dead simply disappears.
+    void fuse_copies(Forwarding& fwd) {
+        for (const auto& r : cr_)
+            if (!(r.d.flags & DEVOP_VEC) || (r.d.bytes & 15u) || (r.d.flags >> DEVOP_HEAD_SHIFT & 15u)) return;
+        std::vector<char> removed(nrows(), 0);
+        bool any = false;
+        for (const auto& cc : plan_.comps) {
+            for (uint32_t p = cc.row_first; p < cc.row_end; ++p) {
+                if (removed[p] || !(fwd.flags[p] & DEVOP_PUT)) continue;
+                const uint32_t k = fwd.slots[p] >> 16 & 0xffu;
+                std::vector<uint32_t> extra;
+                for (uint32_t q = p + 1; q < cc.row_end; ++q) {
+                    if (removed[q]) continue;
+                    if ((fwd.flags[q] & DEVOP_PUT) && (fwd.slots[q] >> 16 & 0xffu) == k) break;       // the slot gets another value
+                    const ColRow& c = cr_[q];
+                    if (c.d.kind != SAR_OP_COPY || !(fwd.flags[q] & DEVOP_GET1) || (fwd.slots[q] >> 8 & 0xffu) != k || c.d.bytes != cr_[p].d.bytes) continue;
+                    bool clean = true;                    // nobody touches the destination between the two rows
+                    for (auto it = first_after(c.c0, p); it != ev_[(size_t)c.c0].end() && it->row < q; ++it) clean = false;
+                    if (!clean) continue;
+                    removed[q] = 1; any = true;
+                    if (!(fwd.flags[q] & DEVOP_DEAD0)) extra.push_back(q);
+                }
+                if (extra.empty()) continue;
+                ColRow& pr = cr_[p];
+                const uint32_t first = (uint32_t)ptrs_.size();
+                if (pr.d.kind == SAR_OP_MREDUCE) {        // its list again, with the new destinations behind the old
+                    if (fwd.flags[p] & DEVOP_DEAD0) {     // ... which go when their store was dead: the flag covers the whole list
+                        pr.d.ndst = 0; pr.mwrites.clear(); fwd.flags[p] &= ~(uint32_t)DEVOP_DEAD0;
+                    }
+                    for (uint32_t i = 0; i < pr.d.nsrc + pr.d.ndst; ++i) { char* const t = ptrs_[pr.d.ptr_off + i]; ptrs_.push_back(t); }
+                } else if (pr.d.ndst) {
+                    for (uint32_t i = 0; i < pr.d.ndst; ++i) { char* const t = ptrs_[pr.d.ptr_off + i]; ptrs_.push_back(t); }
+                }
+                for (uint32_t q : extra) { ptrs_.push_back(cr_[q].d.p0); pr.mwrites.push_back(cr_[q].c0); }
+                pr.d.ptr_off = first; pr.d.ndst += (uint32_t)extra.size();
+            }
+        }
+        if (any) remove_rows(removed, fwd);
     }
 
     // Stores nobody needs.  A row's result for a cell is dead when a later row overwrites the cell and every row

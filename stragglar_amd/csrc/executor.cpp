@@ -75,7 +75,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -541,7 +541,7 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
-           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1) &&
+           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1) && t.col_fuse_copies >= 0 && t.col_fuse_copies <= 2 &&
            (t.arena_spread == 0 || t.arena_spread == 1);
 }
 
@@ -1087,6 +1087,7 @@ int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, i
                 } else {
                     locate(d.p0, &r.dst_rank, &r.dst_off);
                     locate(d.p1, &r.src_rank, &r.src_off);
+                    r.ndst = (int32_t)d.ndst; r.first_ptr = (int32_t)d.ptr_off;      // extra destinations
                 }
                 out_rows[i] = r;
             }

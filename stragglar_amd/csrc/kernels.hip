@@ -508,6 +508,8 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                                     if (live0) st16<SNT>(p0 + o, s);
                                     if (kind == SAR_OP_XREDUCE && live1) st16<SNT>(p1 + o, s);
                                     if (FWD && (flags & DEVOP_PUT)) mine[((slots >> 16 & 0xffu) * V + v) * BLOCK] = s;
+                                    // copies of the result that later rows would have made (taken over by the host)
+                                    if (FWD && row.ndst) { char* const* const more = ptrs + row.ptr_off; for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(more[d] + o, s); }
                                 }
                             }
                         }

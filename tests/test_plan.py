@@ -89,14 +89,20 @@ def test_small_messages_take_the_plan_for_few_items(sarlib):
     st = plan(sarlib, "stragglar", 8, S)
     assert st.executor == 1 and st.launches == 1 and st.col_block == 256 and st.col_components == 7
     assert st.col_slots == 1                                  # broadcast trees keep forwarding there
+    # halving-doubling: half its rows still load, which alone would not pay; but the doubling half are copies of
+    # held values that the reducing rows can store themselves, and with those gone it does
     rhd = plan(sarlib, "rhd", 8, S)
-    assert rhd.executor == 1 and rhd.col_slots == 0           # rows that mostly still load do not
+    assert rhd.executor == 1 and rhd.col_slots == 4
+    assert plan(sarlib, "rhd", 8, S, col_fuse_copies=0).col_slots == 0
     assert plan(sarlib, "rhd", 8, S, col_latency_plan=0).col_slots == 4
+    rows, _ = sarlib.plan_rows(sarlib.builtin("rhd", 8), 8, S)
+    assert len(rows) == 8 * 7 and all(r.kind == 2 for r in rows) and sum(r.ndst for r in rows) == 8 * 7
     # ring: the reduce-scatter chain of a chunk becomes one multi-source row, and what is left are copies of its result
     ring = plan(sarlib, "ring", 8, S)
     assert ring.executor == 1 and ring.col_slots == 1
-    assert plan(sarlib, "ring", 8, S, col_fuse_chains=0).col_slots == 0
-    rows, ptrs = sarlib.plan_rows(sarlib.builtin("ring", 8), 8, S)
+    assert plan(sarlib, "ring", 8, S, col_fuse_chains=0).col_slots == 1           # the all-gather's copies go into the last reducing row
+    assert plan(sarlib, "ring", 8, S, col_fuse_chains=0, col_fuse_copies=0).col_slots == 0
+    rows, ptrs = sarlib.plan_rows(sarlib.builtin("ring", 8), 8, S, col_fuse_copies=0)
     assert [r.kind for r in rows if r.component == 0] == [3] + [0] * 7
     first = rows[0]
     assert (first.nsrc, first.ndst, first.put_slot, first.dead0) == (8, 1, 0, 0)
@@ -104,6 +110,18 @@ def test_small_messages_take_the_plan_for_few_items(sarlib):
     chunk = S // 8
     c = ptrs[first.first_ptr][1] // chunk
     assert [rank for rank, _ in ptrs[first.first_ptr:first.first_ptr + 9]] == [(c + 1 + k) % 8 for k in range(8)] + [c]
+    # and the all-gather's copies of that result are stores of the same row: one row per chunk, 8 sources, 8 destinations
+    rows, ptrs = sarlib.plan_rows(sarlib.builtin("ring", 8), 8, S)
+    assert len(rows) == 8 and all((r.kind, r.nsrc, r.ndst) == (3, 8, 8) for r in rows)
+    first = rows[0]
+    c = ptrs[first.first_ptr][1] // chunk
+    assert sorted(rank for rank, _ in ptrs[first.first_ptr + 8:first.first_ptr + 16]) == list(range(8))
+    assert all(off == c * chunk for _, off in ptrs[first.first_ptr:first.first_ptr + 16])
+    # the StragglAR table: an exchange and the six copies of its broadcast tree are one row with six more destinations
+    rows, ptrs = sarlib.plan_rows(sarlib.builtin("stragglar", 8), 8, S)
+    assert len(rows) == 7 and all((r.kind, r.nsrc, r.ndst) == (1, 0, 6) for r in rows)
+    for r in rows:
+        assert sorted([r.dst_rank, r.src_rank] + [rank for rank, _ in ptrs[r.first_ptr:r.first_ptr + 6]]) == list(range(8))
 
 
 def test_prework_and_misaligned_buffers(sarlib):
@@ -198,7 +216,7 @@ def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
                 slots[(r.component, r.put_slot)] = acc
             continue
         if not r.vector:
-            assert r.head_bytes == 0 and r.get0_slot < 0 and r.get1_slot < 0 and r.put_slot < 0 and not r.dead0 and not r.dead1
+            assert r.head_bytes == 0 and r.get0_slot < 0 and r.get1_slot < 0 and r.put_slot < 0 and not r.dead0 and not r.dead1 and r.ndst == 0
             through_memory(r, r.dst_off, r.src_off, r.bytes)
             continue
         assert r.dst_off % 16 == 0 and r.src_off % 16 == 0
@@ -220,12 +238,16 @@ def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
         if r.kind == 1 and not r.dead1:
             src[:] = s
         assert r.kind == 1 or not r.dead1
+        for rank, off in ptrs[r.first_ptr:r.first_ptr + r.ndst]:        # copies of the result taken over from later rows
+            assert vec == r.bytes and r.head_bytes == 0
+            view(rank, off, off + vec)[:] = s
         if r.put_slot >= 0:
             slots[(r.component, r.put_slot)] = s.copy()
 
 
-PLAN_SETTINGS = [dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_slots=1), dict(col_latency_plan=0, col_slots=3),
-                 dict(col_latency_plan=2, col_slots=8), dict(col_forward=0), dict(col_split=0, col_slots=4), dict(col_latency_plan=0, col_elide_stores=0)]
+PLAN_SETTINGS = [dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_slots=1), dict(col_latency_plan=0, col_slots=3, col_fuse_copies=2),
+                 dict(col_latency_plan=2, col_slots=8), dict(col_forward=0), dict(col_split=0, col_slots=4), dict(col_latency_plan=0, col_elide_stores=0),
+                 dict(col_fuse_copies=0), dict(col_latency_plan=2, col_slots=2, col_fuse_copies=0, col_fuse_chains=0), dict(col_latency_plan=0, col_slots=8, col_fuse_copies=2)]
 
 
 @pytest.mark.parametrize("dtype,chunk_elems", [("f32", 1024), ("f32", 4 * 37 + 1), ("bf16", 8 * 50), ("f16", 8 * 21 + 3)])
@@ -269,7 +291,7 @@ def test_plan_with_the_prework_in_the_same_launch_carried_out_on_the_cpu(sarlib,
                 assert_bits_equal(got[r], want[r], "n=%d %s settings %r rank %d" % (n, dtype, t, r))
 
 
-@pytest.mark.parametrize("seed", range(150))
+@pytest.mark.parametrize("seed", range(400))
 def test_plans_of_random_row_lists_carried_out_on_the_cpu(sarlib, oracle, seed):
     import numpy as np
     from conftest import apply_row_list, assert_bits_equal, make_inputs, random_row_list
@@ -289,6 +311,73 @@ def test_plans_of_random_row_lists_carried_out_on_the_cpu(sarlib, oracle, seed):
         carry_out_plan(oracle, rows, ptrs, got, dtype)
         for r in range(n):
             assert_bits_equal(got[r], want[r], "seed %d settings %r rank %d\n%s" % (seed, t, r, text))
+
+
+def test_copies_of_a_result_whose_own_store_is_dead(sarlib, oracle):
+    """A chain of one-sided reduces that became one multi-source row, whose store is dead (rank 1 chunk 2 is
+    overwritten later) while a copy of its result to another rank (rank 2 chunk 5) is not: the row must drop its
+    own destination and keep the copy.  (A table a random search found.)"""
+    import numpy as np
+    from conftest import apply_row_list, assert_bits_equal, make_inputs
+    text = """sar-rows 4 6
+round
+copy 0 2 2 1 3
+xreduce 1 3 0 3
+round
+xreduce 2 0 3 2
+reduce 0 1 1 2 1
+xreduce 0 2 0 1
+round
+reduce 2 1 0 2 1
+reduce 2 0 5 5 1
+xreduce 3 1 4 1
+round
+reduce 3 1 4 0 1
+round
+xreduce 1 0 0 2
+copy 0 3 3 0 3
+xreduce 1 3 3 3
+round
+reduce 1 3 2 4 1
+xreduce 1 0 3 2
+reduce 2 0 1 1 1
+round
+reduce 3 1 0 1 1
+reduce 0 1 1 2 3
+xreduce 2 3 1 2
+round
+copy 1 2 2 5 1
+reduce 1 2 0 0 2
+round
+reduce 2 3 3 0 1
+reduce 3 1 4 1 2
+reduce 1 2 5 1 1
+copy 3 0 5 1 1
+"""
+    table = []
+    for line in text.splitlines()[1:]:
+        w = line.split()
+        if w[0] == "round":
+            table.append([])
+        elif w[0] == "xreduce":
+            table[-1].append(("xreduce", int(w[1]), int(w[2]), int(w[3]), int(w[3]), int(w[4])))
+        else:
+            table[-1].append((w[0], int(w[1]), int(w[2]), int(w[3]), int(w[4]), int(w[5])))
+    n, parts, dtype, elems = 4, 6, "bf16", 6 * 64 + 2
+    main = sarlib.parse(text, n)
+    inputs = make_inputs(n, elems, dtype, seed=8321, kind="ints")
+    want = [x.copy() for x in inputs]
+    apply_row_list(oracle, table, want, parts, dtype)
+    for t in (dict(col_split=0, col_slots=3), dict(col_latency_plan=2, col_slots=1), dict(col_split=0, col_slots=3, col_fuse_copies=0)):
+        rows, ptrs = sarlib.plan_rows(main, n, elems * 2, dtype, executor=1, **t)
+        got = [x.copy() for x in inputs]
+        carry_out_plan(oracle, rows, ptrs, got, dtype)
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "settings %r rank %d" % (t, r))
+    rows, ptrs = sarlib.plan_rows(main, n, elems * 2, dtype, executor=1, col_split=0, col_slots=3)
+    fused = [r for r in rows if r.kind == 3]
+    assert len(fused) == 1 and fused[0].dead0 == 0 and fused[0].ndst == 1
+    assert ptrs[fused[0].first_ptr + fused[0].nsrc] == (2, 5 * 128)
 
 
 def test_plan_rows_errors(sarlib):
