@@ -161,13 +161,14 @@ def main():
     mean_launch_bytes = statistics.fmean(launch_bytes)
     achieved = mean_launch_bytes / mean_launch_ms / 1e6
     traffic = None
+    traffic_table = {}
     tpath = os.path.join(ROOT, "profiles", "kernel_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            t = json.load(f)
+            traffic_table = json.load(f)
         key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, ("column_forwarding" if st.col_slots else "column") if st.executor == 1 else "rounds")
-        if key in t:
-            traffic = t[key]["hbm_bytes_per_launch"]
+        if key in traffic_table:
+            traffic = traffic_table[key]["hbm_bytes_per_launch"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                 "kernel": "sar::column_kernel<f32, %d, %s>" % (st.col_block, "forwarding" if st.col_slots else "no forwarding") if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
@@ -217,10 +218,10 @@ def main():
                                        "frac_of_hbm_peak": round(st.algorithmic_bytes / pm / 1e6 / HBM_PEAK_GBPS, 4),
                                        "ranks_identical_after_run": bool(ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts))}
         plain_key = "%s_n%d_%dMiB_f32_column" % (args.alg, n, args.mib)
-        if os.path.exists(tpath) and plain_key in t:
+        if plain_key in traffic_table:
             # what the counters saw of it: re-reads of an item that hit the XCD's own L2 never reach the fabric
-            rec["every_operand_loaded"]["traffic"] = t[plain_key]["hbm_bytes_per_launch"]
-            rec["every_operand_loaded"]["memory_side_GBps"] = round(t[plain_key]["hbm_bytes_per_launch"] / pm / 1e6, 1)
+            rec["every_operand_loaded"]["traffic"] = traffic_table[plain_key]["hbm_bytes_per_launch"]
+            rec["every_operand_loaded"]["memory_side_GBps"] = round(traffic_table[plain_key]["hbm_bytes_per_launch"] / pm / 1e6, 1)
         ctx.set_tuning(col_forward=1)
         ctx.prepare(main_sched, None, use_graph=False)
     if not args.no_cpu and args.alg == "stragglar":
