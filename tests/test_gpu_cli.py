@@ -82,3 +82,42 @@ def test_reducescatter_twin():
     for i, l in enumerate(lines):
         m = re.match(r"^1053696,(\d+),(\d+\.\d{3}),(\d+\.\d{3})$", l)
         assert m and int(m.group(1)) == i + 1
+
+
+@pytest.mark.parametrize("extra", [[], ["--executor", "0"], ["--forward", "0"], ["--alg", "ring", "--no-cpu"]])
+def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
+    """bench.py end to end (at 16 MiB per rank so that it takes a second): exactly one JSON line on stdout, the
+    keys the harness reads, a roofline object and, for the StragglAR run, the CPU baseline."""
+    import json
+    import sys
+    p = run(sys.executable, os.path.join(ROOT, "bench.py"), "--mib", "16", "--steps", "3", "--warmup", "1", *extra)
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = [l for l in p.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1, p.stdout
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+                "dtype", "data", "config", "roofline"):
+        assert key in rec, key
+    assert rec["unit"] == "GB/s" and rec["n_gpus"] == 1 and rec["steps"] == 3 and rec["warmup"] == 1 and rec["vs_baseline"] is None
+    assert rec["dtype"] == "f32" and rec["higher_is_better"] is True and "workload" in rec["config"] and rec["value"] > 0
+    roof = rec["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s" and "traffic" in roof
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    assert rec["ranks_identical_after_run"] is True
+    if "--no-cpu" not in extra:
+        base = rec["cpu_baseline"]
+        assert base["kind"] == "port" and base["cores"] == 1 and base["value"] > 0 and base["unit"] == "GB/s" and base["sample"]
+        assert rec["bit_exact_vs_cpu_checker"] is True
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import sys
+    p = run(sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2")
+    assert p.returncode != 0 and "--gpus" in p.stderr and p.stdout.strip() == ""
+
+
+def test_smoke_entry_point():
+    """__graft_entry__.smoke(): one small AllReduce through the HIP library, checked against the CPU checker."""
+    import sys
+    p = run(sys.executable, "-c", "import sys; sys.path.insert(0, %r); import __graft_entry__ as g; g.smoke()" % ROOT)
+    assert p.returncode == 0 and "smoke ok" in p.stdout, p.stdout + p.stderr
