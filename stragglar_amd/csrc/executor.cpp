@@ -164,9 +164,10 @@ bool find_spread_pair(sar_ctx* c, uint64_t bytes) {
     if (free_b < 4 * bytes + kSpreadHeadroom) return false;
     // enough candidates to cross a region boundary from anywhere, no more
     const uint64_t budget = std::min<uint64_t>((uint64_t)free_b - kSpreadHeadroom, kSpreadSearch + 2 * bytes);
+    std::vector<char*> held;
+    try { held.reserve((size_t)(budget / bytes) + 1); } catch (const std::bad_alloc&) { return false; }      // no allocation below
     char* lo = nullptr;
     if (hipMalloc((void**)&lo, bytes) != hipSuccess) { (void)hipGetLastError(); return false; }
-    std::vector<char*> held;
     char* hi = nullptr;
     for (uint64_t used = bytes; used + bytes <= budget; used += bytes) {
         char* cand = nullptr;
