@@ -50,6 +50,7 @@ enum {
 };
 
 #define SAR_MAX_RANKS 64
+#define SAR_MAX_RANK_BYTES (1ull << 40)   /* largest bytes_per_rank any call accepts */
 
 typedef struct sar_ctx sar_ctx;
 typedef struct sar_schedule sar_schedule;
@@ -218,7 +219,10 @@ void sar_destroy(sar_ctx* ctx);
 
 /* Rank buffers, replacing cudaMallocAsync(d_buffers[i]) (allreduce_8GPU.cu
  * :977-990).  No temp buffers exist: exchanges are fused.  All ranks share one
- * arena; rank r starts at r*stride, stride = bytes rounded up to 2 MiB. */
+ * arena; rank r starts at r*stride, stride = bytes rounded up to 2 MiB (with
+ * tuning.arena_spread the upper half of the ranks starts over in a second
+ * allocation).  bytes_per_rank: a positive multiple of the element size, at
+ * most SAR_MAX_RANK_BYTES. */
 int sar_alloc_ranks(sar_ctx* ctx, int n, uint64_t bytes_per_rank, int dtype);
 
 /* Use caller-owned device buffers as the rank buffers instead of the arena: device_ptrs[r] is rank r's

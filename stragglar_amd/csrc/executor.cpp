@@ -46,6 +46,14 @@ struct Launch {
 
 int elem_size_of(int dtype) { return dtype == SAR_F32 ? 4 : 2; }
 
+// Runs the body of an entry point; no exception leaves the C ABI.
+template <class F> int guarded(F&& body) {
+    try { return body(); }
+    catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory"); }
+    catch (const std::exception& e) { return set_error(SAR_EINVAL, e.what()); }
+    catch (...) { return set_error(SAR_EINVAL, "unexpected error"); }
+}
+
 }  // namespace
 
 // A column plan as it sits on the device.
@@ -562,6 +570,7 @@ struct HostPlan {
         if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
         if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
         if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+    if (bytes_per_rank > SAR_MAX_RANK_BYTES) return set_error(SAR_EINVAL, "bytes_per_rank is larger than SAR_MAX_RANK_BYTES");
         if (tuning && !valid_tuning(*tuning)) return set_error(SAR_EINVAL, "tuning value out of range");
         for (const sar_schedule* s : {prework, main_sched}) {
             if (!s) continue;
@@ -618,13 +627,17 @@ int sar_schedule_builtin(const char* alg, int n, sar_schedule** out) {
     } catch (const std::exception& e) { return set_error(SAR_EINVAL, e.what()); }
 }
 
-int sar_schedule_validate(const sar_schedule* s, char* msg, size_t cap) {
+static int schedule_validate_body(const sar_schedule* s, char* msg, size_t cap) {
     if (!s) return set_error(SAR_EINVAL, "schedule is null");
     std::string why;
     try { why = sar::validate(s->s); } catch (const std::exception& e) { why = e.what(); }
     if (msg && cap) { std::snprintf(msg, cap, "%s", why.c_str()); }
     if (!why.empty()) return set_error(SAR_ESCHED, why);
     return SAR_OK;
+}
+
+int sar_schedule_validate(const sar_schedule* s, char* msg, size_t cap) {
+    return guarded([&] { return schedule_validate_body(s, msg, cap); });
 }
 
 int sar_schedule_ranks(const sar_schedule* s) { return s ? s->s.n : SAR_EINVAL; }
@@ -706,11 +719,12 @@ void sar_destroy(sar_ctx* c) {
     delete c;
 }
 
-int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
+static int alloc_ranks_body(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
     if (!c) return set_error(SAR_EINVAL, "context is null");
     if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
     if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
     if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+    if (bytes_per_rank > SAR_MAX_RANK_BYTES) return set_error(SAR_EINVAL, "bytes_per_rank is larger than SAR_MAX_RANK_BYTES");
     SAR_HIP(hipSetDevice(c->device));
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_ranks(c);
@@ -741,12 +755,17 @@ int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
     return SAR_OK;
 }
 
-int sar_adopt_ranks(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
+int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
+    return guarded([&] { return alloc_ranks_body(c, n, bytes_per_rank, dtype); });
+}
+
+static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
     if (!c) return set_error(SAR_EINVAL, "context is null");
     if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
     if (!device_ptrs) return set_error(SAR_EINVAL, "pointer list is null");
     if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
     if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
+    if (bytes_per_rank > SAR_MAX_RANK_BYTES) return set_error(SAR_EINVAL, "bytes_per_rank is larger than SAR_MAX_RANK_BYTES");
     SAR_HIP(hipSetDevice(c->device));
     for (int r = 0; r < n; ++r) {
         if (!device_ptrs[r]) return set_error(SAR_EINVAL, "a rank pointer is null");
@@ -766,6 +785,10 @@ int sar_adopt_ranks(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_
     for (int r = 0; r < n; ++r) c->adopted.push_back((char*)device_ptrs[r]);
     c->n = n; c->dtype = dtype; c->bytes_per_rank = bytes_per_rank; c->stride = 0;
     return SAR_OK;
+}
+
+int sar_adopt_ranks(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
+    return guarded([&] { return adopt_ranks_body(c, n, device_ptrs, bytes_per_rank, dtype); });
 }
 
 static int check_rank_range(sar_ctx* c, int rank, uint64_t off, uint64_t bytes) {
@@ -804,7 +827,7 @@ int sar_fill_const(sar_ctx* c, int rank, uint64_t elem_off, uint64_t elems, doub
     return SAR_OK;
 }
 
-int sar_fill_reference_pattern(sar_ctx* c, const char* alg, float delay_ms, int base) {
+static int fill_reference_pattern_body(sar_ctx* c, const char* alg, float delay_ms, int base) {
     if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (!alg) return set_error(SAR_EINVAL, "alg is null");
     const std::string a(alg);
@@ -822,6 +845,10 @@ int sar_fill_reference_pattern(sar_ctx* c, const char* alg, float delay_ms, int 
     }
     SAR_HIP(hipStreamSynchronize(c->stream));
     return SAR_OK;
+}
+
+int sar_fill_reference_pattern(sar_ctx* c, const char* alg, float delay_ms, int base) {
+    return guarded([&] { return fill_reference_pattern_body(c, alg, delay_ms, base); });
 }
 
 static int fill_random(sar_ctx* c, int rank, uint64_t seed, double a, double b, int mode) {
@@ -894,7 +921,7 @@ int sar_set_tuning(sar_ctx* c, const sar_tuning_t* in) {
     c->tune = *in; return SAR_OK;
 }
 
-int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph) {
+static int prepare_body(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph) {
     if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (!main_sched) return set_error(SAR_EINVAL, "main schedule is null");
     for (const sar_schedule* s : {prework, main_sched}) {
@@ -941,6 +968,10 @@ int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* mai
     return SAR_OK;
 }
 
+int sar_prepare(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, int use_graph) {
+    return guarded([&] { return prepare_body(c, prework, main_sched, use_graph); });
+}
+
 int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
     if (!(delay_ms <= kMaxDelayMs)) return set_error(SAR_EINVAL, "delay out of range");
@@ -975,7 +1006,7 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     return SAR_OK;
 }
 
-int sar_run_profiled(sar_ctx* c, float* ms, int cap, int* count) {
+static int run_profiled_body(sar_ctx* c, float* ms, int cap, int* count) {
     if (!c || !c->prepared) return set_error(SAR_ESTATE, "sar_prepare has not succeeded");
     if (cap < 0 || (cap > 0 && !ms)) return set_error(SAR_EINVAL, "bad argument");
     SAR_HIP(hipSetDevice(c->device));
@@ -1003,6 +1034,10 @@ int sar_run_profiled(sar_ctx* c, float* ms, int cap, int* count) {
     for (size_t i = 0; i < ls.size() && (int)i < cap; ++i) SAR_HIP(hipEventElapsedTime(&ms[i], c->ev_prof[i], c->ev_prof[i + 1]));
     if (count) *count = (int)ls.size();
     return SAR_OK;
+}
+
+int sar_run_profiled(sar_ctx* c, float* ms, int cap, int* count) {
+    return guarded([&] { return run_profiled_body(c, ms, cap, count); });
 }
 
 int sar_launch_bytes(sar_ctx* c, uint64_t* bytes, int cap, int* count) {
@@ -1041,7 +1076,7 @@ int sar_default_tuning(sar_tuning_t* out) {
     *out = sar_ctx().tune; return SAR_OK;
 }
 
-int sar_plan(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+static int plan_body(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
              const sar_tuning_t* tuning, int compute_units, sar_stats_t* out) {
     if (!out) return set_error(SAR_EINVAL, "null argument");
     HostPlan hp;
@@ -1051,7 +1086,12 @@ int sar_plan(const sar_schedule* prework, const sar_schedule* main_sched, int n,
     return SAR_OK;
 }
 
-int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+int sar_plan(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+             const sar_tuning_t* tuning, int compute_units, sar_stats_t* out) {
+    return guarded([&] { return plan_body(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units, out); });
+}
+
+static int plan_rows_body(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
                   const sar_tuning_t* tuning, int compute_units, int same_launch,
                   sar_plan_row* out_rows, int row_cap, int* nrows, sar_plan_ptr* out_ptrs, int ptr_cap, int* nptrs) {
     if (!nrows || !nptrs || (row_cap > 0 && !out_rows) || (ptr_cap > 0 && !out_ptrs) || row_cap < 0 || ptr_cap < 0)
@@ -1095,6 +1135,12 @@ int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, i
         }
     }
     return SAR_OK;
+}
+
+int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
+                  const sar_tuning_t* tuning, int compute_units, int same_launch,
+                  sar_plan_row* out_rows, int row_cap, int* nrows, sar_plan_ptr* out_ptrs, int ptr_cap, int* nptrs) {
+    return guarded([&] { return plan_rows_body(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units, same_launch, out_rows, row_cap, nrows, out_ptrs, ptr_cap, nptrs); });
 }
 
 }  // extern "C"

@@ -390,3 +390,15 @@ def test_plan_rows_errors(sarlib):
         sarlib.plan_rows(sarlib.builtin("stragglar", 8), 8, S, same_launch=True)              # no pre-work given
     with pytest.raises(sa.SarError):
         sarlib.plan_rows(sarlib.builtin("direct", 8), 8, S, prework=sarlib.builtin("prework_ar", 8), same_launch=True)   # chunking differs
+
+
+def test_rank_size_limit(sarlib):
+    """Sizes whose 2 MiB rounding or rank multiple would wrap 64 bits are refused, not planned."""
+    import stragglar_amd as sa
+    main = sarlib.builtin("ring", 8)
+    for S in ((1 << 40) + 4, (1 << 64) - 4):
+        with pytest.raises(sa.SarError) as ei:
+            sarlib.plan_rows(main, 8, S)
+        assert ei.value.code == -1 and "SAR_MAX_RANK_BYTES" in str(ei.value)
+    st = sarlib.plan(main, 8, 1 << 40)                   # the limit itself plans
+    assert st.algorithmic_bytes == 35 * (1 << 40)
