@@ -43,17 +43,17 @@ __device__ __forceinline__ void st16(char* p, f4 v) {
 // ---- element arithmetic ---------------------------------------------------
 // fp32: IEEE add.  fp16: correctly rounded add (same bits as widening to
 // fp32, adding, and narrowing with round-to-nearest-even).  bf16: widen by a
-// shift, fp32 add, round-to-nearest-even narrow, NaN quieted.
-__device__ __forceinline__ uint32_t bf16_round(float f) {
-    uint32_t x = __float_as_uint(f);
-    uint32_t r = (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;
-    uint32_t q = (x >> 16) | 0x40u;
-    return ((x & 0x7fffffffu) > 0x7f800000u) ? q : r;
-}
+// shift, fp32 add, round-to-nearest-even narrow by gfx950's v_cvt_pk_bf16_f32
+// (two results per instruction; the integer sequence it replaces cost 18 VALU
+// operations per pair against 7 and showed in schedules that add a lot).  A NaN
+// stays a NaN; which NaN is the hardware's choice.
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+typedef float f2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t bf16x2_add(uint32_t a, uint32_t b) {
-    float lo = __uint_as_float(a << 16) + __uint_as_float(b << 16);
-    float hi = __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u);
-    return (bf16_round(lo) & 0xffffu) | (bf16_round(hi) << 16);
+    f2 s;
+    s.x = __uint_as_float(a << 16) + __uint_as_float(b << 16);
+    s.y = __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(s, bf2));
 }
 
 template <int DT>
@@ -79,8 +79,7 @@ template <> struct Elem<SAR_BF16> { typedef uint16_t T; };
 template <int DT>
 __device__ __forceinline__ typename Elem<DT>::T add1(typename Elem<DT>::T a, typename Elem<DT>::T b) {
     if constexpr (DT == SAR_BF16) {
-        float s = __uint_as_float((uint32_t)a << 16) + __uint_as_float((uint32_t)b << 16);
-        return (uint16_t)bf16_round(s);
+        return (uint16_t)bf16x2_add(a, b);
     } else {
         return a + b;
     }
@@ -602,6 +601,14 @@ hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, h
 }
 
 // ---- fills -------------------------------------------------------------------
+
+// fp32 -> bf16, round to nearest even, NaN quieted (fills are not hot: plain integer code)
+__device__ __forceinline__ uint32_t bf16_round(float f) {
+    uint32_t x = __float_as_uint(f);
+    uint32_t r = (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;
+    uint32_t q = (x >> 16) | 0x40u;
+    return ((x & 0x7fffffffu) > 0x7f800000u) ? q : r;
+}
 
 __device__ __forceinline__ uint16_t narrow16(float f, int dtype) {
     if (dtype == SAR_F16) { _Float16 h = (_Float16)f; return __builtin_bit_cast(uint16_t, h); }

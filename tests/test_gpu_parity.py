@@ -196,6 +196,39 @@ def test_special_values(gpu_ctx, sarlib, oracle):
                 assert np.array_equal(got[r][~nan], want[r][~nan]), (dtype, r)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_every_16_bit_pattern_as_an_operand(gpu_ctx, sarlib, oracle, dtype):
+    """Every one of the 65536 bit patterns of a 16-bit type added to 96 partners (zeros, the smallest and largest
+    finite values, subnormals, infinities, values that round up to the next binade or overflow, and random ones):
+    the rounding of the sum must be the checker's in every case, ties and subnormal results included.  NaN
+    results only have to be NaNs."""
+    rng = np.random.default_rng(11)
+    special = {"f16": [0x0000, 0x8000, 0x0001, 0x8001, 0x03ff, 0x0400, 0x7bff, 0xfbff, 0x7c00, 0xfc00, 0x3c00, 0xbc00, 0x3bff, 0x7800, 0x0200, 0x8200],
+               "bf16": [0x0000, 0x8000, 0x0001, 0x8001, 0x007f, 0x0080, 0x7f7f, 0xff7f, 0x7f80, 0xff80, 0x3f80, 0xbf80, 0x3f7f, 0x7f00, 0x0040, 0x8040]}[dtype]
+    partners = np.array(special + list(rng.integers(0, 65536, 96 - len(special))), dtype=np.uint16)
+    a = np.tile(np.arange(65536, dtype=np.uint16), partners.size)
+    b = np.repeat(partners, 65536)
+    text = "sar-rows 2 1\nround\nreduce 1 0 0 0\nround\nxreduce 0 1 0\n"       # a += b (one-sided), then s = a + b on both sides
+    main = sarlib.parse(text, 2)
+    want = [a.copy(), b.copy()]
+    apply_row_list(oracle, [[("reduce", 1, 0, 0, 0, 1)], [("xreduce", 1, 0, 0, 0, 1)]], want, 1, dtype)
+    ctx = gpu_ctx
+    ctx.alloc_ranks(2, a.size * 2, dtype)
+    for t in (dict(executor=1), dict(executor=0), dict(executor=1, col_forward=0)):
+        ctx.set_tuning(**dict(ctx.default_tuning, **t))
+        ctx.upload(0, a); ctx.upload(1, b)
+        ctx.prepare(main, None)
+        ctx.run(-1.0)
+        for r in range(2):
+            got = ctx.download(r)
+            g, w = from_bits(got, dtype), from_bits(want[r], dtype)
+            nan = np.isnan(g) & np.isnan(w)
+            assert np.array_equal(np.isnan(g), np.isnan(w)), (dtype, t, r)
+            bad = np.flatnonzero((got != want[r]) & ~nan)
+            assert bad.size == 0, "%s %r rank %d: %d differ, first a=%#06x b=%#06x got %#06x want %#06x" % (
+                dtype, t, r, bad.size, a[bad[0]], b[bad[0]], got[bad[0]], want[r][bad[0]])
+
+
 def test_every_tuning_gives_the_same_bits(gpu_ctx, sarlib, oracle):
     n, dtype = 8, "f32"
     nbytes = sarlib.pad_bytes(300000, n) + 4 * 3          # a partial last tile and a 3-element tail
