@@ -138,8 +138,10 @@ typedef struct sar_tuning_t {
                           /*     (in the plan for few work items, where the round trips are the cost) */
     int32_t col_fuse_copies; /* column executor: 1 = copies of a value that an earlier row of the work   */
                           /*     item still holds are issued by that row as extra stores, and the    */
-                          /*     copy rows (with their round boundaries) go away, in the plan for    */
-                          /*     few work items; 2 = in every plan; 0 = never                       */
+                          /*     copy rows (with their round boundaries) go away, where that was     */
+                          /*     measured to pay: the plan for few work items, payloads up to 768    */
+                          /*     MiB, plans whose value slots limit the workgroups per CU;           */
+                          /*     2 = in every plan; 0 = never                                        */
     int32_t arena_spread; /* sar_alloc_ranks: 1 = for payloads of 128 MiB and more, half the ranks go   */
                           /*     into an allocation of their own that a short timing probe has shown */
                           /*     to lie in another region of HBM than the first half's (MI355X:     */

@@ -55,7 +55,7 @@ public:
         }
         const bool pays = !plan_.staged || env_.tune.col_slots != 0 || !fwd.nslots || slots_pay_when_staged(fwd);
         const uint32_t rows_before = (uint32_t)before.cr.size();
-        if (fwd.nslots && (env_.tune.col_fuse_copies == 2 || (env_.tune.col_fuse_copies == 1 && plan_.staged))) fuse_copies(fwd);
+        if (fwd.nslots && (env_.tune.col_fuse_copies == 2 || (env_.tune.col_fuse_copies == 1 && copies_pay(fwd)))) fuse_copies(fwd);
         // (latency plan) ... or when taking the copies of held values into the rows that produce them shortens the
         // items by a quarter or more (halving-doubling: the doubling half disappears, 11.4 -> 10.2 us at n = 8)
         if (!pays && nrows() * 4u > rows_before * 3u) {
@@ -359,6 +359,19 @@ private:
     // chain).  Keep it when two thirds of the rows are such (the broadcast trees of the StragglAR tables and of
     // direct: n = 32 at 1 MiB per rank 17.8 us against 21.8 us; ring once its reduce-scatter chain is one row),
     // not for rows that mostly still load (halving-doubling: 12.9 against 11.7 us at n = 8).
+    // Copies stored by the row that produced their value (col_fuse_copies = 1): always in the latency plan.  In the
+    // bandwidth plan the traffic is the same either way and what is saved is rows, which counts while a good part of
+    // the payload stays in the 256 MB Infinity Cache (n = 8: 3 to 9 % faster at 8 to 64 MiB per rank, equal to 3 %
+    // slower at 256 MiB, where eight stores in one burst suit the memory less than stores spread over the rounds),
+    // and where the value slots leave a CU fewer workgroups than its thread limit allows, so that the rows of an item
+    // have less company to hide behind (halving-doubling, 4 or 5 slots: 3 % faster at every size).
+    bool copies_pay(const Forwarding& fwd) const {
+        if (plan_.staged) return true;
+        if (env_.bytes_per_rank * (uint64_t)env_.n <= (768ull << 20)) return true;
+        const uint64_t wgs_by_threads = 2048u / (uint32_t)plan_.block;
+        return (uint64_t)fwd.nslots * column_bytes(plan_.block, true) * wgs_by_threads > column_lds_budget();
+    }
+
     bool slots_pay_when_staged(const Forwarding& fwd) const {
         uint32_t free_rows = 0;
         for (uint32_t i = 0; i < nrows(); ++i) free_rows += cr_[i].d.kind == SAR_OP_COPY && (fwd.flags[i] & DEVOP_GET1);
