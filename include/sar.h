@@ -330,7 +330,8 @@ typedef struct sar_plan_row {
     int32_t ndst;        /* ... and destinations: entries [first_ptr, first_ptr + nsrc + ndst) of the pointer   */
     int32_t first_ptr;   /* list.  Other kinds: nsrc = 0 and ndst further destinations of the result (copies    */
                          /* of it that later rows would have made), entries [first_ptr, first_ptr + ndst)       */
-    int32_t reserved;
+    int32_t joins;       /* 1 = (plan for few work items) the row takes its operands together with the row      */
+                         /* before it, ahead of that row's sum and stores                                       */
 } sar_plan_row;
 
 typedef struct sar_plan_ptr { int32_t rank; int32_t reserved; uint64_t off; } sar_plan_ptr;

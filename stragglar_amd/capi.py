@@ -51,7 +51,7 @@ class PlanRow(ctypes.Structure):
                 ("dst_rank", ctypes.c_int32), ("src_rank", ctypes.c_int32), ("dst_off", ctypes.c_uint64), ("src_off", ctypes.c_uint64),
                 ("bytes", ctypes.c_uint64), ("head_bytes", ctypes.c_int32), ("get0_slot", ctypes.c_int32), ("get1_slot", ctypes.c_int32),
                 ("put_slot", ctypes.c_int32), ("dead0", ctypes.c_int32), ("dead1", ctypes.c_int32), ("nsrc", ctypes.c_int32),
-                ("ndst", ctypes.c_int32), ("first_ptr", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("ndst", ctypes.c_int32), ("first_ptr", ctypes.c_int32), ("joins", ctypes.c_int32)]
 
 
 class PlanPtr(ctypes.Structure):

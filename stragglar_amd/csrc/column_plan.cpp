@@ -64,6 +64,7 @@ public:
         }
         plan_.nslots = fwd.nslots; plan_.forwarded_bytes = fwd.bytes;
         for (uint32_t i = 0; i < nrows(); ++i) { cr_[i].d.flags |= fwd.flags[i]; cr_[i].d.slots = fwd.slots[i]; }
+        if (plan_.staged) mark_joins();
         choose_launch();
         for (const auto& r : cr_) { rows.push_back(r.d); plan_.multi_source |= r.d.kind == SAR_OP_MREDUCE; }
         return SAR_OK;
@@ -546,6 +547,32 @@ private:
             if (r.c0 == r.c1) continue;
             if (dead(i, r.c0)) { fwd.flags[i] |= DEVOP_DEAD0; plan_.elided_bytes += vec_bytes; }
             if (r.d.kind == SAR_OP_XREDUCE && dead(i, r.c1)) { fwd.flags[i] |= DEVOP_DEAD1; plan_.elided_bytes += vec_bytes; }
+        }
+    }
+
+    // Plan for few work items: nothing covers a row's round trip to memory there, and the rows of a group do not
+    // depend on each other through memory.  Runs of up to four whole-vector rows of a group take their operands
+    // together (DEVOP_JOIN on every row of a run but the first).  Two rows of a group can still meet in a value
+    // slot -- both read the same cell and the first one keeps it for the second -- so a row that takes a slot which
+    // a row of the run fills starts a run of its own.
+    void mark_joins() {
+        constexpr uint32_t kRun = 4;
+        for (size_t g = 0; g + 1 < plan_.group_begin.size(); ++g) {
+            uint32_t start = plan_.group_begin[g];
+            bool start_plain = false;
+            for (uint32_t i = plan_.group_begin[g]; i < plan_.group_begin[g + 1]; ++i) {
+                DevOp& d = cr_[i].d;
+                const bool plain = (d.flags & DEVOP_VEC) && d.kind != SAR_OP_MREDUCE;
+                bool join = i > plan_.group_begin[g] && plain && start_plain && i - start < kRun;
+                for (uint32_t p = start; p < i && join; ++p) {
+                    const DevOp& e = cr_[p].d;
+                    if (!(e.flags & DEVOP_PUT)) continue;
+                    const uint32_t k = e.slots >> 16 & 0xffu;
+                    if (((d.flags & DEVOP_GET0) && (d.slots & 0xffu) == k) || ((d.flags & DEVOP_GET1) && (d.slots >> 8 & 0xffu) == k)) join = false;
+                }
+                if (join) d.flags |= DEVOP_JOIN;
+                else { start = i; start_plain = plain; }
+            }
         }
     }
 

@@ -1122,6 +1122,7 @@ static int plan_rows_body(const sar_schedule* prework, const sar_schedule* main_
                 r.get1_slot = (d.flags & sar::DEVOP_GET1) ? (int32_t)(d.slots >> 8 & 0xffu) : -1;
                 r.put_slot = (d.flags & sar::DEVOP_PUT) ? (int32_t)(d.slots >> 16 & 0xffu) : -1;
                 r.dead0 = (d.flags & sar::DEVOP_DEAD0) ? 1 : 0; r.dead1 = (d.flags & sar::DEVOP_DEAD1) ? 1 : 0;
+                r.joins = (d.flags & sar::DEVOP_JOIN) ? 1 : 0;
                 if (d.kind == SAR_OP_MREDUCE) {
                     r.dst_rank = r.src_rank = -1;
                     r.nsrc = (int32_t)d.nsrc; r.ndst = (int32_t)d.ndst; r.first_ptr = (int32_t)d.ptr_off;

@@ -387,6 +387,50 @@ static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offset
               offsetof(DevOp, flags) == 28 && offsetof(DevOp, nsrc) == 40 && offsetof(DevOp, ndst) == 44 &&
               offsetof(DevOp, ptr_off) == 48 && offsetof(DevOp, slots) == 52, "column_row reads DevOp by position");
 
+// Latency plan (one vector per lane and row), a row of whole vectors in two steps, so that the loads of several
+// rows of a group can be in flight together: the rows of a group never depend on each other.
+template <int BLOCK, bool FWD, bool LNT>
+__device__ __forceinline__ void lat_row_load(const ColRow& row, uint64_t voff, const f4* mine, f4& a, f4& b) {
+    a = f4{0.f, 0.f, 0.f, 0.f}; b = a;
+    if (voff + 16u > row.bytes) return;
+    const uint32_t slots = FWD ? row.slots : 0u;
+    if (FWD && (row.flags & DEVOP_GET1)) b = mine[(slots >> 8 & 0xffu) * BLOCK]; else b = ld16<LNT>(row.p1 + voff);
+    if (row.kind != SAR_OP_COPY) { if (FWD && (row.flags & DEVOP_GET0)) a = mine[(slots & 0xffu) * BLOCK]; else a = ld16<LNT>(row.p0 + voff); }
+}
+
+template <int DT, int BLOCK, bool FWD, bool SNT>
+__device__ __forceinline__ void lat_row_finish(const ColRow& row, uint64_t off, uint64_t voff, f4* mine, char* const* __restrict__ ptrs, f4 a, f4 b) {
+    typedef typename Elem<DT>::T T;
+    const uint32_t flags = row.flags, kind = row.kind;
+    char* const p0 = row.p0;
+    char* const p1 = row.p1;
+    if (voff + 16u <= row.bytes) {
+        const f4 s = kind == SAR_OP_COPY ? b : add16<DT>(a, b);
+        if (!(FWD && (flags & DEVOP_DEAD0))) st16<SNT>(p0 + voff, s);
+        if (kind == SAR_OP_XREDUCE && !(FWD && (flags & DEVOP_DEAD1))) st16<SNT>(p1 + voff, s);
+        if (FWD && (flags & DEVOP_PUT)) mine[(row.slots >> 16 & 0xffu) * BLOCK] = s;
+        if (FWD && row.ndst) { char* const* const more = ptrs + row.ptr_off; for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(more[d] + voff, s); }
+    }
+    // the bytes behind the last whole vector and in front of the first one, as in the one-row path
+    const uint64_t tail_at = row.bytes & ~(uint64_t)15u;
+    const uint32_t tail = (uint32_t)(row.bytes & 15u) / sizeof(T);
+    if (tail && tail_at >= off && tail_at < off + (uint64_t)BLOCK * 16u && threadIdx.x < tail) {
+        const uint64_t o = tail_at + threadIdx.x * sizeof(T);
+        T s = *reinterpret_cast<const T*>(p1 + o);
+        if (kind != SAR_OP_COPY) s = add1<DT>(*reinterpret_cast<const T*>(p0 + o), s);
+        *reinterpret_cast<T*>(p0 + o) = s;
+        if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
+    }
+    const uint32_t head = (flags >> DEVOP_HEAD_SHIFT & 15u) / (uint32_t)sizeof(T);
+    if (head && off == 0 && threadIdx.x < head) {
+        const int64_t o = ((int64_t)threadIdx.x - (int64_t)head) * (int64_t)sizeof(T);
+        T s = *reinterpret_cast<const T*>(p1 + o);
+        if (kind != SAR_OP_COPY) s = add1<DT>(*reinterpret_cast<const T*>(p0 + o), s);
+        *reinterpret_cast<T*>(p0 + o) = s;
+        if (kind == SAR_OP_XREDUCE) *reinterpret_cast<T*>(p1 + o) = s;
+    }
+}
+
 // Rows that share no (rank, chunk) cell never depend on each other, whatever round they sit in.  The host
 // therefore splits the rows into connected components (for all four algorithms: one per chunk index) and a
 // work item is one component for one column: its rows, in round order, cut into groups at the round
@@ -448,6 +492,30 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
             else { rb = group_begin[g]; re = group_begin[g + 1u]; }
             for (uint32_t j = rb; j < re; ++j) {
                 const ColRow row = column_row<LAT>(ops, table, j);
+                if (LAT && j + 1u < re) {
+                    // Few items: nothing covers a row's round trip to memory.  Rows that the host flagged DEVOP_JOIN
+                    // (up to three behind a row of whole vectors, none needing another's result) go together: all
+                    // their loads and slot reads first, then the sums and stores in row order.
+                    constexpr uint32_t K = 4;
+                    ColRow rw[K];
+                    rw[0] = row;
+                    uint32_t nb = 1;
+#pragma unroll
+                    for (uint32_t q = 1; q < K; ++q)
+                        if (nb == q && j + q < re) {
+                            rw[q] = column_row<true>(ops, table, j + q);
+                            if (rw[q].flags & DEVOP_JOIN) nb = q + 1u;
+                        }
+                    if (nb > 1u) {
+                        f4 a[K], b[K];
+#pragma unroll
+                        for (uint32_t q = 0; q < K; ++q) if (q < nb) lat_row_load<BLOCK, FWD, LNT>(rw[q], voff, mine, a[q], b[q]);
+#pragma unroll
+                        for (uint32_t q = 0; q < K; ++q) if (q < nb) lat_row_finish<DT, BLOCK, FWD, SNT>(rw[q], off, voff, mine, ptrs, a[q], b[q]);
+                        j += nb - 1u;
+                        continue;
+                    }
+                }
                 const uint32_t flags = row.flags, kind = row.kind;
                 const uint64_t bytes = row.bytes;
                 char* const p0 = row.p0;

@@ -20,6 +20,9 @@ enum : uint32_t {
                            // overwritten before anybody loads them (every reader in between takes the value from
                            // a slot): not stored
     DEVOP_DEAD1 = 4096u,   // the same for p1 (XREDUCE)
+    DEVOP_JOIN = 8192u,    // column executor, plan for few work items: the row takes its operands together with the
+                           // row before it (same group; it needs neither that row's result nor that of any row
+                           // the one before joined), and the sums and stores follow in row order
     DEVOP_HEAD_SHIFT = 8u  // column executor: flags >> 8 & 15 = bytes of the row that lie before p0 and p1 (both moved
                            // up to the next 16-byte boundary; `bytes` counts from there)
 };

@@ -97,6 +97,11 @@ def test_small_messages_take_the_plan_for_few_items(sarlib):
     assert plan(sarlib, "rhd", 8, S, col_latency_plan=0).col_slots == 4
     rows, _ = sarlib.plan_rows(sarlib.builtin("rhd", 8), 8, S)
     assert len(rows) == 8 * 7 and all(r.kind == 2 for r in rows) and sum(r.ndst for r in rows) == 8 * 7
+    # the four reduces of a chunk's first round load eight cold operands: they take them together (and the two of
+    # the second round their slot values); nowhere else are there two rows in a group
+    for c in range(8):
+        assert [(r.group, r.joins) for r in rows if r.component == c] == [(0, 0), (0, 1), (0, 1), (0, 1), (1, 0), (1, 1), (2, 0)]
+    assert not any(r.joins for r in sarlib.plan_rows(sarlib.builtin("rhd", 8), 8, sarlib.pad_bytes(256 << 20, 8))[0])    # plan for many items: one row at a time
     # ring: the reduce-scatter chain of a chunk becomes one multi-source row, and what is left are copies of its result
     ring = plan(sarlib, "ring", 8, S)
     assert ring.executor == 1 and ring.col_slots == 1
@@ -178,6 +183,9 @@ ES = {"f32": 4, "f16": 2, "bf16": 2}
 
 
 def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
+    """The planned rows on numpy arrays, the way the column kernel runs them: component by component, group by
+    group, row by row, except that a row and the rows behind it that are flagged `joins` first take all their
+    operands, from memory or from slots, and only then add and store in row order."""
     es = ES[dtype]
     slots = {}
 
@@ -197,41 +205,39 @@ def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
             oracle.reduce_add(dst, src, dtype)
             src[:] = dst
 
-    last = (-1, -1)
-    for r in rows:
-        assert (r.component, r.group) >= last, "rows come component by component, group by group"
-        last = (r.component, r.group)
-        if r.kind == 3:
-            assert r.vector and r.bytes % 16 == 0 and r.head_bytes == 0
-            srcs, dsts = ptrs[r.first_ptr:r.first_ptr + r.nsrc], ptrs[r.first_ptr + r.nsrc:r.first_ptr + r.nsrc + r.ndst]
-            acc = view(srcs[0][0], srcs[0][1], srcs[0][1] + r.bytes).copy()
-            for rank, off in srcs[1:]:
-                t = view(rank, off, off + r.bytes).copy()
-                oracle.reduce_add(t, acc, dtype)                 # the next source + what has been summed so far
-                acc = t
-            if not r.dead0:
-                for rank, off in dsts:
-                    view(rank, off, off + r.bytes)[:] = acc
-            if r.put_slot >= 0:
-                slots[(r.component, r.put_slot)] = acc
-            continue
-        if not r.vector:
-            assert r.head_bytes == 0 and r.get0_slot < 0 and r.get1_slot < 0 and r.put_slot < 0 and not r.dead0 and not r.dead1 and r.ndst == 0
-            through_memory(r, r.dst_off, r.src_off, r.bytes)
-            continue
+    def multi_source(r):
+        assert r.vector and r.bytes % 16 == 0 and r.head_bytes == 0
+        srcs, dsts = ptrs[r.first_ptr:r.first_ptr + r.nsrc], ptrs[r.first_ptr + r.nsrc:r.first_ptr + r.nsrc + r.ndst]
+        acc = view(srcs[0][0], srcs[0][1], srcs[0][1] + r.bytes).copy()
+        for rank, off in srcs[1:]:
+            t = view(rank, off, off + r.bytes).copy()
+            oracle.reduce_add(t, acc, dtype)                 # the next source + what has been summed so far
+            acc = t
+        if not r.dead0:
+            for rank, off in dsts:
+                view(rank, off, off + r.bytes)[:] = acc
+        if r.put_slot >= 0:
+            slots[(r.component, r.put_slot)] = acc
+
+    def take_operands(r):
         assert r.dst_off % 16 == 0 and r.src_off % 16 == 0
         vec = r.bytes & ~15
-        through_memory(r, r.dst_off - r.head_bytes, r.src_off - r.head_bytes, r.head_bytes)
-        through_memory(r, r.dst_off + vec, r.src_off + vec, r.bytes - vec)
         dst, src = view(r.dst_rank, r.dst_off, r.dst_off + vec), view(r.src_rank, r.src_off, r.src_off + vec)
-        b = slots[(r.component, r.get1_slot)] if r.get1_slot >= 0 else src.copy()
+        b = slots[(r.component, r.get1_slot)].copy() if r.get1_slot >= 0 else src.copy()
         assert b.size == dst.size, "a slot holds a value of another length"
         if r.kind == 0:
             assert r.get0_slot < 0
-            s = b
-        else:
-            s = (slots[(r.component, r.get0_slot)] if r.get0_slot >= 0 else dst).copy()
-            assert s.size == dst.size
+            return None, b
+        a = (slots[(r.component, r.get0_slot)] if r.get0_slot >= 0 else dst).copy()
+        assert a.size == dst.size
+        return a, b
+
+    def finish(r, a, b):
+        vec = r.bytes & ~15
+        dst, src = view(r.dst_rank, r.dst_off, r.dst_off + vec), view(r.src_rank, r.src_off, r.src_off + vec)
+        s = b
+        if r.kind != 0:
+            s = a
             oracle.reduce_add(s, b, dtype)
         if not r.dead0:
             dst[:] = s
@@ -243,6 +249,34 @@ def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
             view(rank, off, off + vec)[:] = s
         if r.put_slot >= 0:
             slots[(r.component, r.put_slot)] = s.copy()
+        through_memory(r, r.dst_off - r.head_bytes, r.src_off - r.head_bytes, r.head_bytes)
+        through_memory(r, r.dst_off + vec, r.src_off + vec, r.bytes - vec)
+
+    last = (-1, -1)
+    for r in rows:
+        assert (r.component, r.group) >= last, "rows come component by component, group by group"
+        last = (r.component, r.group)
+    j = 0
+    while j < len(rows):
+        r = rows[j]
+        run = [r]
+        while j + len(run) < len(rows) and rows[j + len(run)].joins:
+            run.append(rows[j + len(run)])
+        if len(run) > 1:
+            assert len(run) <= 4 and all(q.vector and q.kind != 3 and (q.component, q.group) == (r.component, r.group) for q in run)
+            taken = [take_operands(q) for q in run]
+            for q, (a, b) in zip(run, taken):
+                finish(q, a, b)
+            j += len(run)
+            continue
+        if r.kind == 3:
+            multi_source(r)
+        elif not r.vector:
+            assert r.head_bytes == 0 and r.get0_slot < 0 and r.get1_slot < 0 and r.put_slot < 0 and not r.dead0 and not r.dead1 and r.ndst == 0
+            through_memory(r, r.dst_off, r.src_off, r.bytes)
+        else:
+            finish(r, *take_operands(r))
+        j += 1
 
 
 PLAN_SETTINGS = [dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_slots=1), dict(col_latency_plan=0, col_slots=3, col_fuse_copies=2),
@@ -402,3 +436,19 @@ def test_rank_size_limit(sarlib):
         assert ei.value.code == -1 and "SAR_MAX_RANK_BYTES" in str(ei.value)
     st = sarlib.plan(main, 8, 1 << 40)                   # the limit itself plans
     assert st.algorithmic_bytes == 35 * (1 << 40)
+
+
+def test_rows_that_share_a_cell_do_not_take_their_operands_together(sarlib):
+    """Two copies of one cell in the same round: the second takes the value from the slot the first one fills, so it
+    cannot read that slot before the first has run; independent rows of the round do go together."""
+    text = "sar-rows 4 2\nround\nxreduce 0 1 0\nround\ncopy 0 2 0 0\ncopy 0 3 0 0\ncopy 1 2 1 1\ncopy 1 3 1 1\n"
+    main = sarlib.parse(text, 4)
+    rows, _ = sarlib.plan_rows(main, 4, 2 * 4096, "f32", executor=1, col_fuse_copies=0, col_split=0, col_slots=4)
+    second = [r for r in rows if r.group == 1]
+    assert len(second) == 4
+    for k, r in enumerate(second):
+        fills = {q.put_slot for q in second[:k] if q.put_slot >= 0}
+        run_start = max(i for i in range(k + 1) if not second[i].joins)
+        fills_in_run = {q.put_slot for q in second[run_start:k] if q.put_slot >= 0}
+        assert not (r.joins and ({r.get0_slot, r.get1_slot} & fills_in_run)), (k, fills)
+    assert any(r.joins for r in second)
