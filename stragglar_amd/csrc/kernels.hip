@@ -40,6 +40,11 @@ __device__ __forceinline__ void st16(char* p, f4 v) {
     else *q = v;
 }
 
+// Marks a loaded value as used here, on every path.  A load that some path never uses stays pending in the
+// compiler's bookkeeping, and the next write to its registers -- a slot read, the row table -- then waits for
+// everything in flight, stores included (the memory counter runs in order).
+__device__ __forceinline__ void consume(f4 v) { asm volatile("" : : "v"(v)); }
+
 // ---- element arithmetic ---------------------------------------------------
 // fp32: IEEE add.  fp16: correctly rounded add (same bits as widening to
 // fp32, adding, and narrowing with round-to-nearest-even).  bf16: widen by a
@@ -387,6 +392,19 @@ static_assert(offsetof(DevOp, p1) == 8 && offsetof(DevOp, bytes) == 16 && offset
               offsetof(DevOp, flags) == 28 && offsetof(DevOp, nsrc) == 40 && offsetof(DevOp, ndst) == 44 &&
               offsetof(DevOp, ptr_off) == 48 && offsetof(DevOp, slots) == 52, "column_row reads DevOp by position");
 
+// The sum (or the copied value) of one vector of a row: to the rank buffers, to a value slot, to the further
+// destinations the host attached.  `v`: which of the lane's V vectors.
+template <int DT, int BLOCK, bool FWD, bool SNT, uint32_t V>
+__device__ __forceinline__ void column_row_store(const ColRow& row, uint64_t o, uint32_t v, f4 a, f4 b, bool live0, bool live1, f4* mine,
+                                                 char* const* __restrict__ ptrs) {
+    const f4 s = row.kind == SAR_OP_COPY ? b : add16<DT>(a, b);
+    if (live0) st16<SNT>(row.p0 + o, s);
+    if (row.kind == SAR_OP_XREDUCE && live1) st16<SNT>(row.p1 + o, s);
+    if (FWD && (row.flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = s;
+    // copies of the result that later rows would have made (taken over by the host)
+    if (FWD && row.ndst) { char* const* const more = ptrs + row.ptr_off; for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(more[d] + o, s); }
+}
+
 // Latency plan (one vector per lane and row), a row of whole vectors in two steps, so that the loads of several
 // rows of a group can be in flight together: the rows of a group never depend on each other.
 template <int BLOCK, bool FWD, bool LNT>
@@ -496,22 +514,31 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                     // Few items: nothing covers a row's round trip to memory.  Rows that the host flagged DEVOP_JOIN
                     // (up to three behind a row of whole vectors, none needing another's result) go together: all
                     // their loads and slot reads first, then the sums and stores in row order.
-                    constexpr uint32_t K = 4;
-                    ColRow rw[K];
-                    rw[0] = row;
+                    // (rows and operands in variables of their own, not arrays: see the one-row path below)
+                    ColRow r1 = row, r2 = row, r3 = row;
                     uint32_t nb = 1;
-#pragma unroll
-                    for (uint32_t q = 1; q < K; ++q)
-                        if (nb == q && j + q < re) {
-                            rw[q] = column_row<true>(ops, table, j + q);
-                            if (rw[q].flags & DEVOP_JOIN) nb = q + 1u;
+                    r1 = column_row<true>(ops, table, j + 1u);
+                    if (r1.flags & DEVOP_JOIN) {
+                        nb = 2;
+                        if (j + 2u < re) {
+                            r2 = column_row<true>(ops, table, j + 2u);
+                            if (r2.flags & DEVOP_JOIN) {
+                                nb = 3;
+                                if (j + 3u < re) { r3 = column_row<true>(ops, table, j + 3u); if (r3.flags & DEVOP_JOIN) nb = 4; }
+                            }
                         }
+                    }
                     if (nb > 1u) {
-                        f4 a[K], b[K];
-#pragma unroll
-                        for (uint32_t q = 0; q < K; ++q) if (q < nb) lat_row_load<BLOCK, FWD, LNT>(rw[q], voff, mine, a[q], b[q]);
-#pragma unroll
-                        for (uint32_t q = 0; q < K; ++q) if (q < nb) lat_row_finish<DT, BLOCK, FWD, SNT>(rw[q], off, voff, mine, ptrs, a[q], b[q]);
+                        f4 a0, b0, a1, b1, a2 = f4{0.f, 0.f, 0.f, 0.f}, b2 = a2, a3 = a2, b3 = a2;
+                        lat_row_load<BLOCK, FWD, LNT>(row, voff, mine, a0, b0);
+                        lat_row_load<BLOCK, FWD, LNT>(r1, voff, mine, a1, b1);
+                        if (nb > 2u) lat_row_load<BLOCK, FWD, LNT>(r2, voff, mine, a2, b2);
+                        if (nb > 3u) lat_row_load<BLOCK, FWD, LNT>(r3, voff, mine, a3, b3);
+                        consume(a0); consume(b0); consume(a1); consume(b1); consume(a2); consume(b2); consume(a3); consume(b3);
+                        lat_row_finish<DT, BLOCK, FWD, SNT>(row, off, voff, mine, ptrs, a0, b0);
+                        lat_row_finish<DT, BLOCK, FWD, SNT>(r1, off, voff, mine, ptrs, a1, b1);
+                        if (nb > 2u) lat_row_finish<DT, BLOCK, FWD, SNT>(r2, off, voff, mine, ptrs, a2, b2);
+                        if (nb > 3u) lat_row_finish<DT, BLOCK, FWD, SNT>(r3, off, voff, mine, ptrs, a3, b3);
                         j += nb - 1u;
                         continue;
                     }
@@ -558,27 +585,23 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                             for (uint32_t v = 0; v < V; ++v)
                                 if (live0 && voff + v * vstep + 16u <= bytes) st16<SNT>(p0 + voff + v * vstep, mine[((slots >> 8 & 0xffu) * V + v) * BLOCK]);
                         } else {
-                            f4 a[V], b[V];
-#pragma unroll
-                            for (uint32_t v = 0; v < V; ++v) {
-                                a[v] = f4{0.f, 0.f, 0.f, 0.f};
-                                const uint64_t o = voff + v * vstep;
-                                const uint64_t oc = o + 16u <= bytes ? o : voff;          // past the end: reload the first vector, keep nothing
-                                if (get1) b[v] = mine[((slots >> 8 & 0xffu) * V + v) * BLOCK]; else b[v] = ld16<LNT>(p1 + oc);
-                                if (kind != SAR_OP_COPY) { if (get0) a[v] = mine[((slots & 0xffu) * V + v) * BLOCK]; else a[v] = ld16<LNT>(p0 + oc); }
+                            // (Every operand in a variable of its own: an array of vectors is kept as one wide value,
+                            // and a load into it is waited for on the spot in order to copy it in, which serialises
+                            // the loads of a row.)
+                            const uint64_t o1 = voff + vstep;
+                            const bool in1 = V > 1u && o1 + 16u <= bytes;
+                            const uint64_t oc1 = in1 ? o1 : voff;                  // past the end: reload the first vector, keep nothing
+                            const uint32_t g0 = (slots & 0xffu) * V, g1 = (slots >> 8 & 0xffu) * V;
+                            f4 a0 = f4{0.f, 0.f, 0.f, 0.f}, a1 = a0, b0, b1 = a0;
+                            if (get1) b0 = mine[g1 * BLOCK]; else b0 = ld16<LNT>(p1 + voff);
+                            if (kind != SAR_OP_COPY) { if (get0) a0 = mine[g0 * BLOCK]; else a0 = ld16<LNT>(p0 + voff); }
+                            if (V > 1u) {
+                                if (get1) b1 = mine[(g1 + 1u) * BLOCK]; else b1 = ld16<LNT>(p1 + oc1);
+                                if (kind != SAR_OP_COPY) { if (get0) a1 = mine[(g0 + 1u) * BLOCK]; else a1 = ld16<LNT>(p0 + oc1); }
                             }
-#pragma unroll
-                            for (uint32_t v = 0; v < V; ++v) {
-                                const uint64_t o = voff + v * vstep;
-                                if (o + 16u <= bytes) {
-                                    const f4 s = kind == SAR_OP_COPY ? b[v] : add16<DT>(a[v], b[v]);
-                                    if (live0) st16<SNT>(p0 + o, s);
-                                    if (kind == SAR_OP_XREDUCE && live1) st16<SNT>(p1 + o, s);
-                                    if (FWD && (flags & DEVOP_PUT)) mine[((slots >> 16 & 0xffu) * V + v) * BLOCK] = s;
-                                    // copies of the result that later rows would have made (taken over by the host)
-                                    if (FWD && row.ndst) { char* const* const more = ptrs + row.ptr_off; for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(more[d] + o, s); }
-                                }
-                            }
+                            column_row_store<DT, BLOCK, FWD, SNT, V>(row, voff, 0u, a0, b0, live0, live1, mine, ptrs);
+                            if (V > 1u) { consume(a1); consume(b1); }              // also where the second vector lies past the end
+                            if (V > 1u && in1) column_row_store<DT, BLOCK, FWD, SNT, V>(row, o1, 1u, a1, b1, live0, live1, mine, ptrs);
                         }
                     }
                     // the < 16 bytes behind the last whole vector of the row, in the column that holds them
