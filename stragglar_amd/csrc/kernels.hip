@@ -181,13 +181,29 @@ __device__ __forceinline__ void tile_mreduce(char* const* __restrict__ srcs, uin
         uint32_t i = threadIdx.x + u * BLOCK;
         if (i >= nvec) continue;
         uint64_t o = off + ((uint64_t)i << 4);
+        // (sources in variables of their own and marked used on every path: kept in an array, or left pending on a
+        // path that skips them, they make later register writes wait for everything in flight -- the stores to the
+        // destinations then went out one at a time)
         f4 acc = ld16<LNT>(srcs[0] + o);
         for (uint32_t k0 = 1; k0 < nsrc; k0 += 8) {
-            f4 v[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) if (k0 + j < nsrc) v[j] = ld16<LNT>(srcs[k0 + j] + o);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) if (k0 + j < nsrc) acc = add16<DT>(v[j], acc);
+            const f4 z = f4{0.f, 0.f, 0.f, 0.f};
+            f4 v0 = ld16<LNT>(srcs[k0] + o), v1 = z, v2 = z, v3 = z, v4 = z, v5 = z, v6 = z, v7 = z;
+            if (k0 + 1 < nsrc) v1 = ld16<LNT>(srcs[k0 + 1] + o);
+            if (k0 + 2 < nsrc) v2 = ld16<LNT>(srcs[k0 + 2] + o);
+            if (k0 + 3 < nsrc) v3 = ld16<LNT>(srcs[k0 + 3] + o);
+            if (k0 + 4 < nsrc) v4 = ld16<LNT>(srcs[k0 + 4] + o);
+            if (k0 + 5 < nsrc) v5 = ld16<LNT>(srcs[k0 + 5] + o);
+            if (k0 + 6 < nsrc) v6 = ld16<LNT>(srcs[k0 + 6] + o);
+            if (k0 + 7 < nsrc) v7 = ld16<LNT>(srcs[k0 + 7] + o);
+            consume(acc); consume(v0); consume(v1); consume(v2); consume(v3); consume(v4); consume(v5); consume(v6); consume(v7);
+            acc = add16<DT>(v0, acc);
+            if (k0 + 1 < nsrc) acc = add16<DT>(v1, acc);
+            if (k0 + 2 < nsrc) acc = add16<DT>(v2, acc);
+            if (k0 + 3 < nsrc) acc = add16<DT>(v3, acc);
+            if (k0 + 4 < nsrc) acc = add16<DT>(v4, acc);
+            if (k0 + 5 < nsrc) acc = add16<DT>(v5, acc);
+            if (k0 + 6 < nsrc) acc = add16<DT>(v6, acc);
+            if (k0 + 7 < nsrc) acc = add16<DT>(v7, acc);
         }
         for (uint32_t d = 0; d < ndst; ++d) st16<SNT>(dsts[d] + o, acc);
     }
@@ -561,11 +577,16 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                         if (o + 16u <= bytes) {
                             f4 acc = ld16<LNT>(srcs[0] + o);
                             for (uint32_t k0 = 1; k0 < row.nsrc; k0 += 4u) {
-                                f4 t[4];
-#pragma unroll
-                                for (uint32_t q = 0; q < 4u; ++q) if (k0 + q < row.nsrc) t[q] = ld16<LNT>(srcs[k0 + q] + o);
-#pragma unroll
-                                for (uint32_t q = 0; q < 4u; ++q) if (k0 + q < row.nsrc) acc = add16<DT>(t[q], acc);
+                                const f4 z = f4{0.f, 0.f, 0.f, 0.f};
+                                f4 t0 = ld16<LNT>(srcs[k0] + o), t1 = z, t2 = z, t3 = z;
+                                if (k0 + 1u < row.nsrc) t1 = ld16<LNT>(srcs[k0 + 1u] + o);
+                                if (k0 + 2u < row.nsrc) t2 = ld16<LNT>(srcs[k0 + 2u] + o);
+                                if (k0 + 3u < row.nsrc) t3 = ld16<LNT>(srcs[k0 + 3u] + o);
+                                consume(acc); consume(t0); consume(t1); consume(t2); consume(t3);
+                                acc = add16<DT>(t0, acc);
+                                if (k0 + 1u < row.nsrc) acc = add16<DT>(t1, acc);
+                                if (k0 + 2u < row.nsrc) acc = add16<DT>(t2, acc);
+                                if (k0 + 3u < row.nsrc) acc = add16<DT>(t3, acc);
                             }
                             if (!(FWD && (flags & DEVOP_DEAD0))) for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(dsts[d] + o, acc);
                             if (FWD && (flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = acc;
