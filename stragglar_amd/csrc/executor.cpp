@@ -514,7 +514,23 @@ int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* ma
         // precedes the schedule): its result for a chunk is handed to the exchange of that chunk in a value slot.
         if (columnar && prework && c->tune.col_fuse_prework) {
             *fused_first = (uint32_t)rows.size();
-            if ((rc = lower_column(c, {&prework->s, &main_sched->s}, rows, ptrs, fused)) != SAR_OK) return rc;
+            // A schedule of whole-buffer rows (direct) behind a pre-work that is cut into chunks: the same rows,
+            // written over the pre-work's chunks (the last one takes the elements past the last chunk boundary
+            // along, as the pre-work's last row does).
+            sar::Schedule recut;
+            const sar::Schedule* second = &main_sched->s;
+            if (second->parts == 1 && prework->s.parts > 1) {
+                recut = *second;
+                recut.parts = prework->s.parts;
+                bool whole = true;
+                for (auto& round : recut.rounds)
+                    for (auto& op : round) {
+                        whole = whole && op.kind != SAR_OP_MREDUCE && op.dst_chunk == 0 && op.src_chunk == 0 && op.nchunks == 1;
+                        op.nchunks = recut.parts; op.to_end = 1;
+                    }
+                if (whole) second = &recut;
+            }
+            if ((rc = lower_column(c, {&prework->s, second}, rows, ptrs, fused)) != SAR_OK) return rc;
             *want_fused = rows.size() > *fused_first && !fused.unsupported;
         }
     } catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory"); }

@@ -157,7 +157,7 @@ def test_most_ranks_the_library_takes(gpu_ctx, sarlib, oracle, n):
 
 @pytest.mark.parametrize("executor", [0, 1, 2])
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 8 * 7 * 4 * 13 + 5, 7 * 8 * 2051])
+@pytest.mark.parametrize("elems", [1, 5, 6, 7, 8, 9, 57, 146 * 7, 1000, 4099, 7 * 1024 + 3, 7 * 1024 + 4, 8 * 7 * 4 * 13 + 5, 7 * 8 * 2051])
 def test_ragged_and_unaligned_sizes(gpu_ctx, sarlib, oracle, elems, dtype, executor):
     """Sizes that do not divide by n-1 or n (the tail is never moved, chunk = size/(n-1) as in the
     reference), chunks that are not 16-byte aligned (element-wise path), and buffers shorter than the

@@ -137,8 +137,9 @@ def test_prework_and_misaligned_buffers(sarlib):
     assert plan(sarlib, "stragglar", 8, S, delay=True, col_fuse_prework=0).fused_prework == 0
     assert plan(sarlib, "stragglar", 8, S, delay=True, executor=0).fused_prework == 0
     assert plan(sarlib, "stragglar", 8, S).fused_prework == 0
-    # direct's pre-work cuts the buffer into n-1 chunks, direct itself moves it whole: not merged
-    assert plan(sarlib, "direct", 8, S, delay=True).fused_prework == 0
+    # direct's pre-work cuts the buffer into n-1 chunks, direct itself moves it whole: direct's rows are written over
+    # the pre-work's chunks for the one launch
+    assert plan(sarlib, "direct", 8, S, delay=True).fused_prework == 1
     # chunk of 4k+2 elements: rows keep their alignment only where the chunk offset happens to allow it
     odd = plan(sarlib, "stragglar", 8, 7 * 4 * 1026, col_latency_plan=0)
     assert 0 <= odd.forwarded_bytes < 42 * 4 * 1026
@@ -325,6 +326,34 @@ def test_plan_with_the_prework_in_the_same_launch_carried_out_on_the_cpu(sarlib,
                 assert_bits_equal(got[r], want[r], "n=%d %s settings %r rank %d" % (n, dtype, t, r))
 
 
+@pytest.mark.parametrize("n", [4, 8, 6, 12])
+def test_direct_with_its_prework_in_the_same_launch_carried_out_on_the_cpu(sarlib, oracle, n):
+    """direct moves whole buffers, its (n-1)-rank AllReduce pre-work works chunk by chunk (allreduce_8GPU.cu:115-137):
+    for the one launch direct's rows are cut at the pre-work's chunk boundaries, the last piece taking the elements
+    past the last boundary along.  The pre-work's copies in ranks 1..n-2 are overwritten by the broadcast unread."""
+    from conftest import assert_bits_equal, make_inputs
+    main, pre = sarlib.builtin("direct", n), sarlib.builtin("prework_ar", n)
+    import stragglar_amd as sa
+    with pytest.raises(sa.SarError) as ei:        # a last chunk that is not a whole number of vectors long: separate launches
+        sarlib.plan_rows(main, n, ((n - 1) * 64 + 1) * 4, "f32", prework=pre, same_launch=True, executor=1)
+    assert ei.value.code == -7
+    # (the elements past the last chunk boundary are fewer than n-1: a whole vector of them needs n-1 > 4 in fp32, > 8 in bf16)
+    cases = [("f32", (n - 1) * 256), ("bf16", (n - 1) * 8 * 40)] + ([("f32", (n - 1) * 64 + 4)] if n - 1 > 4 else []) + ([("bf16", (n - 1) * 8 * 40 + 8)] if n - 1 > 8 else [])
+    for dtype, elems in cases:
+        inputs = make_inputs(n, elems, dtype, seed=9)
+        want = [x.copy() for x in inputs]
+        oracle.run("direct", want, dtype, delay=0.0)
+        for t in (dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_fuse_copies=0), dict(col_forward=0)):
+            rows, ptrs = sarlib.plan_rows(main, n, elems * ES[dtype], dtype, prework=pre, same_launch=True, executor=1, **t)
+            assert sum(r.kind == 3 for r in rows) == n - 1 and max(r.component for r in rows) == n - 2
+            if elems % (n - 1) == 0 and t.get("col_forward", 1):
+                assert all(r.dead0 and r.put_slot >= 0 for r in rows if r.kind == 3)
+            got = [x.copy() for x in inputs]
+            carry_out_plan(oracle, rows, ptrs, got, dtype)
+            for r in range(n):
+                assert_bits_equal(got[r], want[r], "n=%d %s elems %d settings %r rank %d" % (n, dtype, elems, t, r))
+
+
 @pytest.mark.parametrize("seed", range(400))
 def test_plans_of_random_row_lists_carried_out_on_the_cpu(sarlib, oracle, seed):
     import numpy as np
@@ -423,7 +452,7 @@ def test_plan_rows_errors(sarlib):
     with pytest.raises(sa.SarError):
         sarlib.plan_rows(sarlib.builtin("stragglar", 8), 8, S, same_launch=True)              # no pre-work given
     with pytest.raises(sa.SarError):
-        sarlib.plan_rows(sarlib.builtin("direct", 8), 8, S, prework=sarlib.builtin("prework_ar", 8), same_launch=True)   # chunking differs
+        sarlib.plan_rows(sarlib.builtin("ring", 8), 8, S, prework=sarlib.builtin("prework_rs", 8), same_launch=True)     # 8 chunks against 7
 
 
 def test_rank_size_limit(sarlib):
