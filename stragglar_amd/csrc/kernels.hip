@@ -613,15 +613,20 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                             const bool in1 = V > 1u && o1 + 16u <= bytes;
                             const uint64_t oc1 = in1 ? o1 : voff;                  // past the end: reload the first vector, keep nothing
                             const uint32_t g0 = (slots & 0xffu) * V, g1 = (slots >> 8 & 0xffu) * V;
-                            f4 a0 = f4{0.f, 0.f, 0.f, 0.f}, a1 = a0, b0, b1 = a0;
-                            if (get1) b0 = mine[g1 * BLOCK]; else b0 = ld16<LNT>(p1 + voff);
-                            if (kind != SAR_OP_COPY) { if (get0) a0 = mine[g0 * BLOCK]; else a0 = ld16<LNT>(p0 + voff); }
-                            if (V > 1u) {
-                                if (get1) b1 = mine[(g1 + 1u) * BLOCK]; else b1 = ld16<LNT>(p1 + oc1);
-                                if (kind != SAR_OP_COPY) { if (get0) a1 = mine[(g0 + 1u) * BLOCK]; else a1 = ld16<LNT>(p0 + oc1); }
-                            }
-                            column_row_store<DT, BLOCK, FWD, SNT, V>(row, voff, 0u, a0, b0, live0, live1, mine, ptrs);
+                            // Slot reads before loads: a slot read that follows a load of the same row in the code is
+                            // made to wait for that load (both may end up in the same registers), and the loads of
+                            // the row would again go out one at a time.
+                            f4 a0 = f4{0.f, 0.f, 0.f, 0.f}, a1 = a0, b0 = a0, b1 = a0;
+                            const bool load_a = kind != SAR_OP_COPY && !get0;
+                            if (get1) { b0 = mine[g1 * BLOCK]; if (V > 1u) b1 = mine[(g1 + 1u) * BLOCK]; }
+                            if (get0 && kind != SAR_OP_COPY) { a0 = mine[g0 * BLOCK]; if (V > 1u) a1 = mine[(g0 + 1u) * BLOCK]; }
+                            if (!get1) { b0 = ld16<LNT>(p1 + voff); if (V > 1u) b1 = ld16<LNT>(p1 + oc1); }
+                            if (load_a) { a0 = ld16<LNT>(p0 + voff); if (V > 1u) a1 = ld16<LNT>(p0 + oc1); }
+                            // (all operands of the row at once, before its first store: a wait placed behind stores
+                            // waits for the stores as well)
+                            consume(a0); consume(b0);
                             if (V > 1u) { consume(a1); consume(b1); }              // also where the second vector lies past the end
+                            column_row_store<DT, BLOCK, FWD, SNT, V>(row, voff, 0u, a0, b0, live0, live1, mine, ptrs);
                             if (V > 1u && in1) column_row_store<DT, BLOCK, FWD, SNT, V>(row, o1, 1u, a1, b1, live0, live1, mine, ptrs);
                         }
                     }
