@@ -376,7 +376,7 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // schedule, and the load is not issued at all.  Every row stores its result to the rank buffers, in
 // schedule order for each element, except where the host found that a later row overwrites the value
 // before anybody loads it (DEVOP_DEAD0 / DEAD1).
-// One row at a time turned out best (24 VGPRs without forwarding, 48 with: eight waves per SIMD
+// One row at a time turned out best (24 VGPRs without forwarding, 38 with: eight waves per SIMD
 // resident, the other workgroups of the compute unit cover a row's latency; batching the loads of
 // several rows cost occupancy and was slower: 6.8 against 7.1 TB/s).
 
@@ -475,8 +475,8 @@ __device__ __forceinline__ void lat_row_finish(const ColRow& row, uint64_t off, 
 // accesses cached, 1 = streaming (nontemporal) loads and cached stores, 2 = streaming loads and stores.  The
 // policy is a template argument because a flavour picked per row at run time does not survive compilation:
 // the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.  MR: the
-// launch has multi-source rows (a pre-work collective in the same launch); their batched loads double the
-// register count, so launches without such rows run a variant without that path.
+// launch has multi-source rows (a pre-work collective in the same launch); their batched loads take more
+// registers and a longer row loop, so launches without such rows run a variant without that path.
 template <int DT, int BLOCK, bool FWD, bool LAT, int POL, bool MR>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
                                                         const ColumnComp* __restrict__ comps, char* const* __restrict__ ptrs, ColumnLaunch L) {
