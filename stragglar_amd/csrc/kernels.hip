@@ -40,6 +40,21 @@ __device__ __forceinline__ void st16(char* p, f4 v) {
     else *q = v;
 }
 
+// One value to `n` destinations whose addresses are a list in memory: the addresses four at a time (one scalar
+// load), so that a long list is not one round trip to the scalar cache per store.
+template <bool NT>
+__device__ __forceinline__ void st16_to_all(char* const* __restrict__ list, uint32_t n, uint64_t o, f4 v) {
+    uint32_t d = 0;
+    for (; d + 4u <= n; d += 4u) {
+        char* const q0 = list[d];
+        char* const q1 = list[d + 1u];
+        char* const q2 = list[d + 2u];
+        char* const q3 = list[d + 3u];
+        st16<NT>(q0 + o, v); st16<NT>(q1 + o, v); st16<NT>(q2 + o, v); st16<NT>(q3 + o, v);
+    }
+    for (; d < n; ++d) st16<NT>(list[d] + o, v);
+}
+
 // Marks a loaded value as used here, on every path.  A load that some path never uses stays pending in the
 // compiler's bookkeeping, and the next write to its registers -- a slot read, the row table -- then waits for
 // everything in flight, stores included (the memory counter runs in order).
@@ -205,7 +220,7 @@ __device__ __forceinline__ void tile_mreduce(char* const* __restrict__ srcs, uin
             if (k0 + 6 < nsrc) acc = add16<DT>(v6, acc);
             if (k0 + 7 < nsrc) acc = add16<DT>(v7, acc);
         }
-        for (uint32_t d = 0; d < ndst; ++d) st16<SNT>(dsts[d] + o, acc);
+        st16_to_all<SNT>(dsts, ndst, o, acc);
     }
     typedef typename Elem<DT>::T T;
     const uint32_t tail = (len & 15u) / sizeof(T);
@@ -418,7 +433,7 @@ __device__ __forceinline__ void column_row_store(const ColRow& row, uint64_t o, 
     if (row.kind == SAR_OP_XREDUCE && live1) st16<SNT>(row.p1 + o, s);
     if (FWD && (row.flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = s;
     // copies of the result that later rows would have made (taken over by the host)
-    if (FWD && row.ndst) { char* const* const more = ptrs + row.ptr_off; for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(more[d] + o, s); }
+    if (FWD && row.ndst) st16_to_all<SNT>(ptrs + row.ptr_off, row.ndst, o, s);
 }
 
 // Latency plan (one vector per lane and row), a row of whole vectors in two steps, so that the loads of several
@@ -443,7 +458,7 @@ __device__ __forceinline__ void lat_row_finish(const ColRow& row, uint64_t off, 
         if (!(FWD && (flags & DEVOP_DEAD0))) st16<SNT>(p0 + voff, s);
         if (kind == SAR_OP_XREDUCE && !(FWD && (flags & DEVOP_DEAD1))) st16<SNT>(p1 + voff, s);
         if (FWD && (flags & DEVOP_PUT)) mine[(row.slots >> 16 & 0xffu) * BLOCK] = s;
-        if (FWD && row.ndst) { char* const* const more = ptrs + row.ptr_off; for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(more[d] + voff, s); }
+        if (FWD && row.ndst) st16_to_all<SNT>(ptrs + row.ptr_off, row.ndst, voff, s);
     }
     // the bytes behind the last whole vector and in front of the first one, as in the one-row path
     const uint64_t tail_at = row.bytes & ~(uint64_t)15u;
@@ -588,7 +603,7 @@ __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__
                                 if (k0 + 2u < row.nsrc) acc = add16<DT>(t2, acc);
                                 if (k0 + 3u < row.nsrc) acc = add16<DT>(t3, acc);
                             }
-                            if (!(FWD && (flags & DEVOP_DEAD0))) for (uint32_t d = 0; d < row.ndst; ++d) st16<SNT>(dsts[d] + o, acc);
+                            if (!(FWD && (flags & DEVOP_DEAD0))) st16_to_all<SNT>(dsts, row.ndst, o, acc);
                             if (FWD && (flags & DEVOP_PUT)) mine[((row.slots >> 16 & 0xffu) * V + v) * BLOCK] = acc;
                         }
                     }
