@@ -215,7 +215,8 @@ void sar_schedule_free(sar_schedule* s);
 /* ---- device context -------------------------------------------------- */
 
 /* Replaces the per-process setup of main() (allreduce_8GPU.cu:939-963): one
- * device, one stream for the ranks that are on time and one for the straggler. */
+ * device, one stream for the schedule (and the straggler's wait in front of it)
+ * and one for the pre-work of the ranks that are on time. */
 int sar_create(int device, sar_ctx** out);
 void sar_destroy(sar_ctx* ctx);
 

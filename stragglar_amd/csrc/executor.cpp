@@ -66,7 +66,7 @@ struct ColumnDevice {
 
 struct sar_ctx {
     int device = 0;
-    hipStream_t stream = nullptr, straggler_stream = nullptr;
+    hipStream_t stream = nullptr, prework_stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr, ev_join = nullptr;
     std::vector<hipEvent_t> ev_prof;
     int wall_khz = 100000;
@@ -473,21 +473,23 @@ int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, Colu
     return SAR_OK;
 }
 
-int launch_one(sar_ctx* c, const Launch& L) {
+int launch_one(sar_ctx* c, const Launch& L, hipStream_t st) {
     if (L.total_tiles == 0) return SAR_OK;
     const uint32_t interleave = (uint32_t)(c->tune.order == 1);
     if (L.mreduce)
-        SAR_HIP(sar::launch_mreduce(c->dtype, c->stream, c->d_ops + L.first_op, L.nops, c->d_ptrs, L.total_tiles, L.tiles_per_op, interleave, L.reverse));
+        SAR_HIP(sar::launch_mreduce(c->dtype, st, c->d_ops + L.first_op, L.nops, c->d_ptrs, L.total_tiles, L.tiles_per_op, interleave, L.reverse));
     else
-        SAR_HIP(sar::launch_round(c->dtype, c->tune.unroll, c->tune.block, c->stream, c->d_ops + L.first_op, L.nops,
+        SAR_HIP(sar::launch_round(c->dtype, c->tune.unroll, c->tune.block, st, c->d_ops + L.first_op, L.nops,
                                   L.total_tiles, L.tiles_per_op, interleave, L.reverse));
     return SAR_OK;
 }
+int launch_one(sar_ctx* c, const Launch& L) { return launch_one(c, L, c->stream); }
 
-int launch_all(sar_ctx* c, const std::vector<Launch>& v) {
-    for (const auto& L : v) { int rc = launch_one(c, L); if (rc) return rc; }
+int launch_all(sar_ctx* c, const std::vector<Launch>& v, hipStream_t st) {
+    for (const auto& L : v) { int rc = launch_one(c, L, st); if (rc) return rc; }
     return SAR_OK;
 }
+int launch_all(sar_ctx* c, const std::vector<Launch>& v) { return launch_all(c, v, c->stream); }
 
 int launch_main(sar_ctx* c) { return c->column ? launch_column_plan(c, c->col) : launch_all(c, c->rounds); }
 
@@ -697,7 +699,7 @@ int sar_create(int device, sar_ctx** out) {
     c->device = device;
     hipError_t e;
     if ((e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking)) != hipSuccess ||
-        (e = hipStreamCreateWithFlags(&c->straggler_stream, hipStreamNonBlocking)) != hipSuccess ||
+        (e = hipStreamCreateWithFlags(&c->prework_stream, hipStreamNonBlocking)) != hipSuccess ||
         (e = hipEventCreate(&c->ev_start)) != hipSuccess || (e = hipEventCreate(&c->ev_stop)) != hipSuccess ||
         (e = hipEventCreateWithFlags(&c->ev_join, hipEventDisableTiming)) != hipSuccess ||
         (e = hipMalloc((void**)&c->d_flag, sizeof(int))) != hipSuccess) {
@@ -722,7 +724,7 @@ void sar_destroy(sar_ctx* c) {
     if (!c) return;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
-    if (c->straggler_stream) (void)hipStreamSynchronize(c->straggler_stream);
+    if (c->prework_stream) (void)hipStreamSynchronize(c->prework_stream);
     drop_ranks(c);
     drop_pair(c);
     for (auto e : c->ev_prof) (void)hipEventDestroy(e);
@@ -731,7 +733,7 @@ void sar_destroy(sar_ctx* c) {
     if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
     if (c->ev_join) (void)hipEventDestroy(c->ev_join);
     if (c->stream) (void)hipStreamDestroy(c->stream);
-    if (c->straggler_stream) (void)hipStreamDestroy(c->straggler_stream);
+    if (c->prework_stream) (void)hipStreamDestroy(c->prework_stream);
     delete c;
 }
 
@@ -1002,12 +1004,16 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
         // nobody is late: pre-work, then the schedule, on one stream
         int rc = launch_all(c, c->prework); if (rc) return rc;
     } else if (delay_ms > 0) {
-        // the straggler's stream is busy for delay_ms while the others do their pre-work
+        // The straggler is busy for delay_ms (gpu_sleep_kernel on its stream, allreduce_8GPU.cu:876-889) while the
+        // others do their pre-work.  Here the wait sits on the stream that goes on to run the schedule and the
+        // pre-work on the second one: a pre-work that hides behind the delay has signalled its event long before
+        // the sleep ends, and the schedule starts right behind the sleep kernel (about 5 us sooner after the
+        // straggler's arrival than with the join of the two streams on the critical path).
         const uint64_t ticks = (uint64_t)((double)delay_ms * (double)c->wall_khz);
-        SAR_HIP(hipStreamWaitEvent(c->straggler_stream, c->ev_start, 0));
-        SAR_HIP(sar::launch_sleep(c->straggler_stream, ticks));
-        SAR_HIP(hipEventRecord(c->ev_join, c->straggler_stream));
-        int rc = launch_all(c, c->prework); if (rc) return rc;
+        SAR_HIP(hipStreamWaitEvent(c->prework_stream, c->ev_start, 0));
+        int rc = launch_all(c, c->prework, c->prework_stream); if (rc) return rc;
+        SAR_HIP(hipEventRecord(c->ev_join, c->prework_stream));
+        SAR_HIP(sar::launch_sleep(c->stream, ticks));
         SAR_HIP(hipStreamWaitEvent(c->stream, c->ev_join, 0));
     }
     if (main_done) {}
@@ -1015,7 +1021,7 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     else { int rc = launch_main(c); if (rc) return rc; }
     SAR_HIP(hipEventRecord(c->ev_stop, c->stream));
     SAR_HIP(hipEventSynchronize(c->ev_stop));
-    if (delay_ms > 0) SAR_HIP(hipStreamSynchronize(c->straggler_stream));
+    if (delay_ms > 0) SAR_HIP(hipStreamSynchronize(c->prework_stream));
     float ms = 0.f;
     SAR_HIP(hipEventElapsedTime(&ms, c->ev_start, c->ev_stop));
     if (elapsed_ms) *elapsed_ms = ms;
