@@ -13,7 +13,7 @@ import sys
 from . import synthesizer_nonpow2, synthesizer_pow2
 from ._synth import table_text
 
-DEFAULT = (4, 6, 8, 12, 16, 32)
+DEFAULT = (4, 6, 8, 12, 16, 24, 32, 48, 64)
 OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "schedules")
 
 
