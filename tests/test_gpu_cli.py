@@ -62,6 +62,17 @@ def test_other_dtypes_and_seeded_inputs():
     assert p.stdout.splitlines()[-1] == "Rank 5, done"
 
 
+@pytest.mark.parametrize("ranks", [12, 24, 64])
+def test_shipped_tables_beyond_the_reference(ranks):
+    """Rank counts the reference has no code for (README.md:35): the driver picks the shipped table for --ranks N
+    and the self-check on the reference's fill pattern (rank i holds i+1) passes: every rank ends with N(N+1)/2."""
+    nbytes = (ranks - 1) * 1024 * 4
+    for delay in ("-1", "0"):
+        p = run(os.path.join(BIN, "allreduce"), str(nbytes), "stragglar", "2", delay, "--ranks", str(ranks))
+        assert p.returncode == 0, p.stdout + p.stderr
+        assert p.stdout.splitlines()[-1] == "Rank %d, done" % (ranks - 1)
+
+
 def test_self_check_failure_aborts_like_the_reference_assert():
     """A size that does not divide by n-1 leaves a tail that is never reduced: the 8-rank reference
     trips assert(hostOut[i] == 36.0); the 4-rank one only prints the mismatches."""
