@@ -236,6 +236,10 @@ int sar_alloc_ranks(sar_ctx* ctx, int n, uint64_t bytes_per_rank, int dtype);
  * work on those buffers against sar_run (which blocks until the result is complete). */
 int sar_adopt_ranks(sar_ctx* ctx, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype);
 
+/* Device address of rank r's buffer (d_buffers[r] of allreduce_8GPU.cu:977-990), for callers that run their own
+ * kernels on the rank buffers or hand them on; valid until the ranks are allocated or adopted anew. */
+int sar_rank_pointer(sar_ctx* ctx, int rank, void** device_ptr);
+
 int sar_upload(sar_ctx* ctx, int rank, uint64_t byte_off, const void* host, uint64_t bytes);
 int sar_download(sar_ctx* ctx, int rank, uint64_t byte_off, void* host, uint64_t bytes);
 
@@ -264,7 +268,9 @@ int sar_restore(sar_ctx* ctx);
 int sar_ranks_identical(sar_ctx* ctx, uint64_t elems, int* identical);
 
 int sar_get_tuning(sar_ctx* ctx, sar_tuning_t* out);
-int sar_set_tuning(sar_ctx* ctx, const sar_tuning_t* in);   /* takes effect at the next sar_prepare */
+/* Takes effect at the next sar_prepare.  A plan prepared under the old values is dropped: sar_run, sar_stats
+ * and the other calls that need a plan return SAR_ESTATE until sar_prepare has run again. */
+int sar_set_tuning(sar_ctx* ctx, const sar_tuning_t* in);
 
 /* Lower `main` (and the optional pre-work run before it in delay mode) onto
  * the allocated ranks: row tables in device memory for the executor the

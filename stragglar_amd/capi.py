@@ -85,6 +85,7 @@ EXPORTS = [
     "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
+    "sar_rank_pointer",
 ]
 
 
@@ -139,6 +140,7 @@ class Library:
             "sar_plan": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, P(Stats)]),
             "sar_plan_rows": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, c_int, P(PlanRow), c_int, P(c_int), P(PlanPtr), c_int, P(c_int)]),
             "sar_default_tuning": (c_int, [P(Tuning)]),
+            "sar_rank_pointer": (c_int, [vp, c_int, P(vp)]),
         }
         assert sorted(sig) == sorted(EXPORTS)
         for name, (res, args) in sig.items():
@@ -302,6 +304,12 @@ class Context:
         arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
         self._c(self._lib.lib.sar_adopt_ranks(self._h, len(device_ptrs), arr, bytes_per_rank, DTYPES[dtype]))
         self.n, self.dtype, self.bytes_per_rank = len(device_ptrs), dtype, bytes_per_rank
+
+    def rank_pointer(self, rank: int) -> int:
+        """Device address of one rank's buffer."""
+        p = ctypes.c_void_p()
+        self._c(self._lib.lib.sar_rank_pointer(self._h, rank, ctypes.byref(p)))
+        return int(p.value)
 
     @property
     def elems(self) -> int:

@@ -91,8 +91,8 @@ struct sar_ctx {
     char** d_ptrs = nullptr;
     std::vector<Launch> prework, rounds;
     sar_stats_t stats{};
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t graph_exec = nullptr;
+    hipGraph_t graph = nullptr, graph_fused = nullptr;            // the main schedule; pre-work + main schedule in one launch
+    hipGraphExec_t graph_exec = nullptr, graph_fused_exec = nullptr;
 
     // column plan (tune.executor == 1): the whole main schedule as one launch
     bool column = false;
@@ -117,6 +117,8 @@ namespace {
 void drop_plan(sar_ctx* c) {
     if (c->graph_exec) { (void)hipGraphExecDestroy(c->graph_exec); c->graph_exec = nullptr; }
     if (c->graph) { (void)hipGraphDestroy(c->graph); c->graph = nullptr; }
+    if (c->graph_fused_exec) { (void)hipGraphExecDestroy(c->graph_fused_exec); c->graph_fused_exec = nullptr; }
+    if (c->graph_fused) { (void)hipGraphDestroy(c->graph_fused); c->graph_fused = nullptr; }
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
     for (ColumnDevice* d : {&c->col, &c->fused}) {
@@ -447,16 +449,12 @@ int launch_column_plan(sar_ctx* c, const ColumnDevice& d) {
     return SAR_OK;
 }
 
-// Copy a column plan's tables to the device (its rows are in d_ops from `first_op` on).
-int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, ColumnDevice& d) {
+// Launch shape of a column plan whose rows sit in the row table from `first_op` on (no device work).
+int shape_column_plan(const sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, ColumnDevice& d) {
     const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
     const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
     const uint64_t items = ncols * cp.comps.size();
     if (items > 0x7fffffffull) return set_error(SAR_EINVAL, "schedule needs more than 2^31 work items");
-    SAR_HIP(hipMalloc((void**)&d.d_group_begin, cp.group_begin.size() * sizeof(uint32_t)));
-    SAR_HIP(hipMemcpy(d.d_group_begin, cp.group_begin.data(), cp.group_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
-    SAR_HIP(hipMalloc((void**)&d.d_comps, cp.comps.size() * sizeof(sar::ColumnComp)));
-    SAR_HIP(hipMemcpy(d.d_comps, cp.comps.data(), cp.comps.size() * sizeof(sar::ColumnComp), hipMemcpyHostToDevice));
     d.block = (uint32_t)cp.block;
     d.slots = cp.nslots;
     d.lane_local = (cp.lane_local && c->tune.col_light_sync) ? 1u : 0u;
@@ -469,6 +467,16 @@ int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, Colu
     d.items = (uint32_t)items;
     const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
     d.grid = (uint32_t)std::min<uint64_t>(items, resident);
+    return SAR_OK;
+}
+
+// Copy a column plan's tables to the device (its rows are in d_ops from `first_op` on).
+int upload_column_plan(sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, ColumnDevice& d) {
+    int rc = shape_column_plan(c, cp, first_op, d); if (rc) return rc;
+    SAR_HIP(hipMalloc((void**)&d.d_group_begin, cp.group_begin.size() * sizeof(uint32_t)));
+    SAR_HIP(hipMemcpy(d.d_group_begin, cp.group_begin.data(), cp.group_begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice));
+    SAR_HIP(hipMalloc((void**)&d.d_comps, cp.comps.size() * sizeof(sar::ColumnComp)));
+    SAR_HIP(hipMemcpy(d.d_comps, cp.comps.data(), cp.comps.size() * sizeof(sar::ColumnComp), hipMemcpyHostToDevice));
     d.ready = true;
     return SAR_OK;
 }
@@ -777,27 +785,43 @@ int sar_alloc_ranks(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtype) {
     return guarded([&] { return alloc_ranks_body(c, n, bytes_per_rank, dtype); });
 }
 
-static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
-    if (!c) return set_error(SAR_EINVAL, "context is null");
+// Caller-owned rank buffers: n device pointers on GPU `device`, element-aligned, each with bytes_per_rank bytes of
+// its allocation in front of it, no two overlapping.  Host checks only; nothing is launched or allocated.
+static int check_rank_pointers(int device, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
     if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
     if (!device_ptrs) return set_error(SAR_EINVAL, "pointer list is null");
     if (dtype != SAR_F32 && dtype != SAR_F16 && dtype != SAR_BF16) return set_error(SAR_EINVAL, "unknown dtype");
     if (bytes_per_rank == 0 || bytes_per_rank % (uint64_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "bytes_per_rank must be a positive multiple of the element size");
     if (bytes_per_rank > SAR_MAX_RANK_BYTES) return set_error(SAR_EINVAL, "bytes_per_rank is larger than SAR_MAX_RANK_BYTES");
-    SAR_HIP(hipSetDevice(c->device));
     for (int r = 0; r < n; ++r) {
         if (!device_ptrs[r]) return set_error(SAR_EINVAL, "a rank pointer is null");
         if ((uintptr_t)device_ptrs[r] % (uintptr_t)elem_size_of(dtype)) return set_error(SAR_EINVAL, "a rank pointer is not aligned to the element size");
         hipPointerAttribute_t at{};
-        if (hipPointerGetAttributes(&at, device_ptrs[r]) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != c->device) {
+        if (hipPointerGetAttributes(&at, device_ptrs[r]) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != device) {
             (void)hipGetLastError();
             return set_error(SAR_EINVAL, "a rank pointer is not device memory of this context's GPU");
         }
+        // the whole of [ptr, ptr + bytes_per_rank) must lie inside the allocation the pointer belongs to: a kernel
+        // that writes past it faults the device instead of returning an error
+        hipDeviceptr_t base = nullptr; size_t span = 0;
+        if (hipMemGetAddressRange(&base, &span, (hipDeviceptr_t)device_ptrs[r]) != hipSuccess) {
+            (void)hipGetLastError();
+            return set_error(SAR_EINVAL, "a rank pointer does not belong to a device allocation");
+        }
+        const uint64_t into = (uint64_t)((const char*)device_ptrs[r] - (const char*)base);
+        if (into > span || bytes_per_rank > span - into) return set_error(SAR_EINVAL, "a rank buffer is shorter than bytes_per_rank");
         for (int q = 0; q < r; ++q) {
             const char* a = (const char*)device_ptrs[q]; const char* b = (const char*)device_ptrs[r];
             if (a < b + bytes_per_rank && b < a + bytes_per_rank) return set_error(SAR_EINVAL, "rank buffers overlap");
         }
     }
+    return SAR_OK;
+}
+
+static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
+    if (!c) return set_error(SAR_EINVAL, "context is null");
+    SAR_HIP(hipSetDevice(c->device));
+    int rc = check_rank_pointers(c->device, n, device_ptrs, bytes_per_rank, dtype); if (rc) return rc;
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_ranks(c);
     for (int r = 0; r < n; ++r) c->adopted.push_back((char*)device_ptrs[r]);
@@ -813,6 +837,13 @@ static int check_rank_range(sar_ctx* c, int rank, uint64_t off, uint64_t bytes) 
     if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
     if (rank < 0 || rank >= c->n) return set_error(SAR_EINVAL, "rank out of range");
     if (off > c->bytes_per_rank || bytes > c->bytes_per_rank - off) return set_error(SAR_EINVAL, "range leaves the rank buffer");
+    return SAR_OK;
+}
+
+int sar_rank_pointer(sar_ctx* c, int rank, void** device_ptr) {
+    int rc = check_rank_range(c, rank, 0, 0); if (rc) return rc;
+    if (!device_ptr) return set_error(SAR_EINVAL, "null argument");
+    *device_ptr = c->rank_base(rank);
     return SAR_OK;
 }
 
@@ -936,6 +967,13 @@ int sar_get_tuning(sar_ctx* c, sar_tuning_t* out) {
 int sar_set_tuning(sar_ctx* c, const sar_tuning_t* in) {
     if (!c || !in) return set_error(SAR_EINVAL, "null argument");
     if (!valid_tuning(*in)) return set_error(SAR_EINVAL, "tuning value out of range");
+    // A prepared plan was lowered for the old values (tile counts, launch shapes, a captured graph): it goes, and
+    // sar_run reports SAR_ESTATE until the next sar_prepare.
+    if (c->prepared) {
+        SAR_HIP(hipSetDevice(c->device));
+        SAR_HIP(hipStreamSynchronize(c->stream));
+        drop_plan(c);
+    }
     c->tune = *in; return SAR_OK;
 }
 
@@ -970,15 +1008,20 @@ static int prepare_body(sar_ctx* c, const sar_schedule* prework, const sar_sched
 
     sar_stats_t st = plan_stats(c, prework, main_sched, cp, c->column, c->fused.ready);
     if (use_graph) {
-        // the main rounds as one graph: kernel nodes only (no memset nodes)
-        hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
-        if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamBeginCapture: ") + hipGetErrorString(e)); }
-        rc = launch_main(c);
-        e = hipStreamEndCapture(c->stream, &c->graph);
-        if (rc != SAR_OK) { drop_plan(c); return rc; }
-        if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e)); }
-        e = hipGraphInstantiate(&c->graph_exec, c->graph, nullptr, nullptr, 0);
-        if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e)); }
+        // the main rounds as one graph, and the single launch of pre-work + schedule (what sar_run with delay 0
+        // runs) as another: kernel nodes only (no memset nodes)
+        for (int which = 0; which < (c->fused.ready ? 2 : 1); ++which) {
+            hipGraph_t* g = which ? &c->graph_fused : &c->graph;
+            hipGraphExec_t* ge = which ? &c->graph_fused_exec : &c->graph_exec;
+            hipError_t e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+            if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamBeginCapture: ") + hipGetErrorString(e)); }
+            rc = which ? launch_column_plan(c, c->fused) : launch_main(c);
+            e = hipStreamEndCapture(c->stream, g);
+            if (rc != SAR_OK) { drop_plan(c); return rc; }
+            if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e)); }
+            e = hipGraphInstantiate(ge, *g, nullptr, nullptr, 0);
+            if (e != hipSuccess) { drop_plan(c); return set_error(SAR_EHIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e)); }
+        }
         st.uses_graph = 1;
     }
     c->stats = st;
@@ -996,9 +1039,10 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
     SAR_HIP(hipSetDevice(c->device));
     SAR_HIP(hipEventRecord(c->ev_start, c->stream));
     bool main_done = false;
-    if (delay_ms == 0 && c->fused.ready && !c->graph_exec) {
+    if (delay_ms == 0 && c->fused.ready) {
         // nobody is late: pre-work and schedule as the one launch planned for this case
-        int rc = launch_column_plan(c, c->fused); if (rc) return rc;
+        if (c->graph_fused_exec) SAR_HIP(hipGraphLaunch(c->graph_fused_exec, c->stream));
+        else { int rc = launch_column_plan(c, c->fused); if (rc) return rc; }
         main_done = true;
     } else if (delay_ms == 0) {
         // nobody is late: pre-work, then the schedule, on one stream
@@ -1167,3 +1211,4 @@ int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, i
 }
 
 }  // extern "C"
+

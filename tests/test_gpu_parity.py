@@ -363,7 +363,9 @@ def test_graph_replays_match_eager(gpu_ctx, sarlib, oracle):
     ctx = gpu_ctx
     ctx.alloc_ranks(n, nbytes, dtype)
     ctx.prepare(sarlib.builtin("stragglar", n), sarlib.builtin("prework_rs", n), use_graph=True)
-    assert ctx.stats().uses_graph == 1
+    st = ctx.stats()
+    # delay 0 replays the graph of the single launch that holds pre-work and schedule
+    assert st.uses_graph == 1 and st.fused_prework == 1
     for rep in range(4):
         for r, x in enumerate(inputs):
             ctx.upload(r, x)                     # eager copies + synchronisation between replays
@@ -503,27 +505,68 @@ def test_error_paths(gpu_ctx, sarlib):
         ctx.close()
 
 
+def test_set_tuning_drops_the_plan(gpu_ctx, sarlib, oracle):
+    """A plan is lowered for the tuning in force at sar_prepare (tile counts, launch shapes).  Changing the tuning
+    afterwards must not run the old plan under the new values: the plan goes and sar_run says so."""
+    import stragglar_amd as sa
+    n, dtype = 8, "f32"
+    nbytes = sarlib.pad_bytes(1 << 20, n)
+    inputs = make_inputs(n, nbytes // 4, dtype, seed=31)
+    want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=-1.0)
+    ctx = gpu_ctx
+    for executor in (0, 1):
+        ctx.alloc_ranks(n, nbytes, dtype)
+        ctx.set_tuning(executor=executor, unroll=8, block=512)
+        ctx.prepare(sarlib.builtin("stragglar", n))
+        ctx.set_tuning(unroll=1, block=256, col_block=256)
+        for call in (ctx.run, ctx.stats, ctx.run_profiled, ctx.launch_bytes):
+            with pytest.raises(sa.SarError) as ei:
+                call()
+            assert ei.value.code == -7
+        ctx.prepare(sarlib.builtin("stragglar", n))
+        for r, x in enumerate(inputs):
+            ctx.upload(r, x)
+        ctx.run(-1.0)
+        for r in range(n):
+            assert_bits_equal(ctx.download(r), want[r], "executor %d rank %d" % (executor, r))
+
+
+def test_adopted_buffers_must_be_long_enough(gpu_ctx, sarlib):
+    """sar_adopt_ranks checks every buffer against the allocation it lies in: a kernel that wrote past it would
+    fault the device, so a short buffer is an error on the host."""
+    import stragglar_amd as sa
+    gpu_ctx.alloc_ranks(2, 1 << 20, "f32")                 # 2 MiB apart in one allocation of 4 MiB
+    ptrs = [gpu_ctx.rank_pointer(r) for r in range(2)]
+    other = sarlib.context(0)
+    try:
+        other.adopt_ranks(ptrs, 1 << 20, "f32")
+        other.adopt_ranks(ptrs, 2 << 20, "f32")
+        with pytest.raises(sa.SarError) as ei:
+            other.adopt_ranks(ptrs, (2 << 20) + 4096, "f32")
+        assert ei.value.code == -1 and "shorter than bytes_per_rank" in ei.value.message
+        with pytest.raises(sa.SarError):
+            other.adopt_ranks([ptrs[0], ptrs[0] + 4096], 1 << 20, "f32")      # overlapping
+    finally:
+        other.close()
+
+
 def gather_slices(ctx, rank, chunk, parts, offs, length):
     """The same `length` elements at each offset of every chunk of one rank, downloaded piecewise."""
     es = ES[ctx.dtype]
     return np.concatenate([ctx.download(rank, (c * chunk + o) * es, length * es) for c in range(parts) for o in offs])
 
 
-@pytest.mark.parametrize("executor", [0, 1])
-def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
-    """Benchmark configuration 2 (the one the headline figure is quoted on) at its real size: n=8, 256 MiB fp32 per rank (2 GiB resident), uniform[-1,1)
-    seeded per rank, stragglar (both tables) / ring / rhd / direct on the same inputs.  Every op is
-    element-wise within chunk structure, so parity is checked on a mini problem gathered from the
-    same positions of every chunk, plus `all ranks identical` over the whole buffers."""
+def full_size_all_algorithms(ctx, sarlib, oracle, executor, nbytes, seed):
+    """n=8 fp32 at a size the checker cannot take whole: stragglar (both tables) / ring / rhd / direct on the same
+    seeded inputs (allreduce_8GPU.cu:1029-1047 dispatches all four at any size).  Every op is element-wise
+    within chunk structure, so parity is checked on a mini problem gathered from the same positions of every
+    chunk, plus `all ranks identical` over the whole buffers."""
     n, dtype = 8, "f32"
-    nbytes = sarlib.pad_bytes(256 << 20, n)
-    assert nbytes == 268441600
     elems = nbytes // 4
-    ctx = gpu_ctx
     ctx.set_tuning(executor=executor)
     ctx.alloc_ranks(n, nbytes, dtype)
     for r in range(n):
-        ctx.fill_uniform(r, 2000 + r, -1.0, 1.0)
+        ctx.fill_uniform(r, seed + r, -1.0, 1.0)
     ctx.snapshot()
     L = 4096
     for alg, table, parts in (("stragglar", read_golden("stragglar_n8_cu.txt"), 7), ("stragglar", shipped_table(8), 7),
@@ -538,6 +581,7 @@ def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
         delay = -1.0 if alg == "direct" else 0.0
         pre = sarlib.builtin("prework_rs", n) if alg == "stragglar" else None
         ctx.prepare(main, pre, use_graph=True)
+        assert ctx.stats().executor == executor
         ctx.run(delay)
         assert ctx.ranks_identical((elems // parts) * parts), alg
         want = run_oracle(oracle, alg, mini_in, dtype, table, delay=delay)
@@ -548,6 +592,24 @@ def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
         total = np.sum([x.astype(np.float64) for x in terms], axis=0)
         mag = np.sum([np.abs(x.astype(np.float64)) for x in terms], axis=0)
         assert np.all(np.abs(got.astype(np.float64) - total) <= 1e-6 * mag)
+
+
+@pytest.mark.parametrize("executor", [0, 1])
+def test_config2_full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor):
+    """Benchmark configuration 2 (the one the headline figure is quoted on) at its real size: n=8, 256 MiB fp32 per
+    rank (2 GiB resident), uniform[-1,1) seeded per rank, the four algorithms on the same inputs."""
+    nbytes = sarlib.pad_bytes(256 << 20, 8)
+    assert nbytes == 268441600
+    full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor, nbytes, seed=2000)
+
+
+@pytest.mark.parametrize("executor", [0, 1])
+def test_config5_1gib_fp32_all_algorithms(gpu_ctx, sarlib, oracle, executor):
+    """Benchmark configuration 5, the largest point of the message-size sweep: n=8, 1 GiB fp32 per rank (8 GiB
+    resident plus the snapshot), stragglar / ring / rhd / direct, both executors."""
+    nbytes = sarlib.pad_bytes(1 << 30, 8)
+    assert nbytes == 1073744896
+    full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor, nbytes, seed=5000)
 
 
 def test_config3_bf16_1gib_with_delay(gpu_ctx, sarlib, oracle):
