@@ -286,6 +286,20 @@ int sar_prepare(sar_ctx* ctx, const sar_schedule* prework, const sar_schedule* m
  * stop.  elapsed_ms is stop - start as in the reference (:1052). */
 int sar_run(sar_ctx* ctx, float delay_ms, float* elapsed_ms);
 
+/* sar_adopt_ranks + sar_prepare + sar_run(delay 0, or < 0 without pre-work) in one call that allocates nothing on the
+ * device.  No counterpart in the reference; it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The row tables that sar_prepare would put in
+ * memory of its own go into an array that is part of the library image, sar_static_scratch_bytes() (1 MiB) per
+ * GPU, held until the process ends; a schedule whose tables need more is refused with SAR_EINVAL (the n = 8
+ * tables take a few KiB, a 64-rank ring about half a MiB).  `stream` is the caller's hipStream_t (NULL = the
+ * null stream): the tables are copied and the kernels launched on it, and the call returns when it has drained
+ * and the result is complete.  device_ptrs as for sar_adopt_ranks (checked the same way); the default tuning
+ * applies.  No context is needed or touched.  All calls on one GPU share the one array, which keeps the last
+ * call's tables: calls that overlap in time on the same GPU race and must be serialised by the caller. */
+int sar_run_static(int device, void* stream, const sar_schedule* prework, const sar_schedule* main_sched, int n,
+                   void* const* device_ptrs, uint64_t bytes_per_rank, int dtype);
+uint64_t sar_static_scratch_bytes(void);
+
 /* Same as sar_run with delay < 0 and no graph, with an event pair around
  * every launch: ms[i] is the duration of launch i (at most cap written,
  * *count = launches). */

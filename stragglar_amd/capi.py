@@ -85,7 +85,7 @@ EXPORTS = [
     "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
-    "sar_rank_pointer",
+    "sar_run_static", "sar_static_scratch_bytes", "sar_rank_pointer",
 ]
 
 
@@ -140,6 +140,8 @@ class Library:
             "sar_plan": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, P(Stats)]),
             "sar_plan_rows": (c_int, [vp, vp, c_int, u64, c_int, P(Tuning), c_int, c_int, P(PlanRow), c_int, P(c_int), P(PlanPtr), c_int, P(c_int)]),
             "sar_default_tuning": (c_int, [P(Tuning)]),
+            "sar_run_static": (c_int, [c_int, vp, vp, vp, c_int, P(vp), u64, c_int]),
+            "sar_static_scratch_bytes": (u64, []),
             "sar_rank_pointer": (c_int, [vp, c_int, P(vp)]),
         }
         assert sorted(sig) == sorted(EXPORTS)
@@ -193,6 +195,13 @@ class Library:
         rows, ptrs = (PlanRow * max(1, nrows.value))(), (PlanPtr * max(1, nptrs.value))()
         self.check(self.lib.sar_plan_rows(*args, rows, nrows.value, ctypes.byref(nrows), ptrs, nptrs.value, ctypes.byref(nptrs)))
         return list(rows)[:nrows.value], [(p.rank, p.off) for p in list(ptrs)[:nptrs.value]]
+
+    def run_static(self, device_ptrs: Sequence[int], bytes_per_rank: int, dtype: str, main: "Schedule",
+                   prework: Optional["Schedule"] = None, device: int = 0, stream: int = 0):
+        """One AllReduce of caller-owned device buffers through the entry point that allocates nothing."""
+        arr = (ctypes.c_void_p * len(device_ptrs))(*device_ptrs)
+        self.check(self.lib.sar_run_static(device, ctypes.c_void_p(stream), prework.handle if prework else None, main.handle,
+                                           len(device_ptrs), arr, bytes_per_rank, DTYPES[dtype]))
 
     def parse(self, text: str, n: int) -> "Schedule":
         raw = text.encode()

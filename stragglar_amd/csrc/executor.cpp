@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -55,6 +56,15 @@ template <class F> int guarded(F&& body) {
 }
 
 }  // namespace
+
+// Row tables of sar_run_static: device memory that belongs to the library image, so that entry point never has to
+// allocate.  Every GPU the library runs on holds its own copy of the array at its own address for the life of the
+// process.  In host code the name is only a handle for hipGetSymbolAddress (static_scratch below); the address it
+// returns is what copies and kernels use.
+#define SAR_STATIC_SCRATCH_BYTES (1u << 20)
+static __device__ __align__(256) unsigned char scratch[SAR_STATIC_SCRATCH_BYTES];
+
+namespace { int static_scratch(int device, char** out); }
 
 // A column plan as it sits on the device.
 struct ColumnDevice {
@@ -724,6 +734,9 @@ int sar_create(int device, sar_ctx** out) {
     }
     int khz = 0;
     if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0) c->wall_khz = khz;
+    // this GPU's address of the static row table (sar_run_static), resolved here once, with the device current
+    char* static_base = nullptr;
+    if (int rc2 = static_scratch(device, &static_base)) { sar_destroy(c); return rc2; }
     *out = c;
     return SAR_OK;
 }
@@ -1212,3 +1225,106 @@ int sar_plan_rows(const sar_schedule* prework, const sar_schedule* main_sched, i
 
 }  // extern "C"
 
+// ---- an entry point that allocates nothing ---------------------------------------------------------------
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+char* g_scratch_ptr[kMaxDevices] = {};      // device address of `scratch` on every GPU it was resolved on
+
+// The address of this GPU's copy of `scratch`, resolved once per device with that device current.
+int static_scratch(int device, char** out) {
+    if (device < 0 || device >= kMaxDevices) return set_error(SAR_EINVAL, "device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        SAR_HIP(hipSetDevice(device));
+        void* p = nullptr;
+        SAR_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return set_error(SAR_EHIP, "hipGetSymbolAddress returned no address for the static row table");
+        g_scratch_ptr[device] = (char*)p;
+    }
+    *out = g_scratch_ptr[device];
+    return SAR_OK;
+}
+
+int run_static_body(int device, void* stream, const sar_schedule* prework, const sar_schedule* main_sched, int n,
+                    void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
+    if (!main_sched) return set_error(SAR_EINVAL, "main schedule is null");
+    int count = 0;
+    int rc = sar_device_count(&count); if (rc) return rc;
+    if (device < 0 || device >= count) return set_error(SAR_EINVAL, "device index out of range");
+    SAR_HIP(hipSetDevice(device));
+    if ((rc = check_rank_pointers(device, n, device_ptrs, bytes_per_rank, dtype)) != SAR_OK) return rc;
+    for (const sar_schedule* s : {prework, main_sched}) {
+        if (!s) continue;
+        if (s->s.n != n) return set_error(SAR_EINVAL, "schedule and rank count disagree");
+        std::string why = sar::validate(s->s);
+        if (!why.empty()) return set_error(SAR_ESCHED, why);
+    }
+    char* base = nullptr;
+    if ((rc = static_scratch(device, &base)) != SAR_OK) return rc;
+
+    // a context that lives on the host only: the caller's buffers and stream, the default tuning, no device objects
+    sar_ctx c;
+    c.device = device; c.stream = (hipStream_t)stream;
+    c.n = n; c.dtype = dtype; c.bytes_per_rank = bytes_per_rank;
+    for (int r = 0; r < n; ++r) c.adopted.push_back((char*)device_ptrs[r]);
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0) c.cu_count = cus;
+    else { (void)hipGetLastError(); c.cu_count = 256; }
+
+    std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
+    ColumnPlan cp, fp; uint32_t col_first = 0, fused_first = 0; bool want_column = false, want_fused = false;
+    if ((rc = plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused)) != SAR_OK) return rc;
+
+    // what runs: pre-work and schedule in one launch, or the pre-work's launches followed by the schedule's (one
+    // column launch, or one launch per round)
+    const bool one_launch = want_column && want_fused;
+    const ColumnPlan* col = one_launch ? &fp : want_column ? &cp : nullptr;
+    const uint32_t col_rows_first = one_launch ? fused_first : col_first;
+    std::vector<Launch> per_round;
+    if (!one_launch) per_round = c.prework;
+    if (!want_column) per_round.insert(per_round.end(), c.rounds.begin(), c.rounds.end());
+
+    // the part of the row table that these launches read
+    uint64_t lo = rows.size(), hi = 0;
+    for (const Launch& L : per_round) if (L.total_tiles) { lo = std::min<uint64_t>(lo, L.first_op); hi = std::max<uint64_t>(hi, (uint64_t)L.first_op + L.nops); }
+    if (col) { lo = std::min<uint64_t>(lo, col_rows_first); hi = std::max<uint64_t>(hi, (uint64_t)col_rows_first + col->group_begin.back()); }
+    if (hi <= lo) return SAR_OK;                // buffers shorter than `parts` elements: nothing moves
+
+    // layout in the static array: [rows][pointer lists][group boundaries][components], each on a 256-byte boundary
+    auto up = [](uint64_t v) { return (v + 255u) & ~(uint64_t)255u; };
+    const uint64_t rows_b = (hi - lo) * sizeof(sar::DevOp), ptrs_b = ptrs.size() * sizeof(char*);
+    const uint64_t grp_b = col ? col->group_begin.size() * sizeof(uint32_t) : 0, comp_b = col ? col->comps.size() * sizeof(sar::ColumnComp) : 0;
+    const uint64_t ptrs_at = up(rows_b), grp_at = ptrs_at + up(ptrs_b), comp_at = grp_at + up(grp_b), need = comp_at + up(comp_b);
+    if (need > SAR_STATIC_SCRATCH_BYTES)
+        return set_error(SAR_EINVAL, "the schedule's row tables take " + std::to_string(need) + " bytes, the static array of sar_run_static holds " +
+                                         std::to_string((uint64_t)SAR_STATIC_SCRATCH_BYTES) + " (use sar_prepare / sar_run)");
+    hipStream_t st = c.stream;
+    SAR_HIP(hipMemcpyAsync(base, rows.data() + lo, rows_b, hipMemcpyHostToDevice, st));
+    if (ptrs_b) SAR_HIP(hipMemcpyAsync(base + ptrs_at, ptrs.data(), ptrs_b, hipMemcpyHostToDevice, st));
+    c.d_ops = (sar::DevOp*)base; c.d_ptrs = (char**)(base + ptrs_at);
+    for (Launch& L : per_round) L.first_op -= (uint32_t)lo;
+    if ((rc = launch_all(&c, per_round, st)) != SAR_OK) { (void)hipStreamSynchronize(st); return rc; }
+    if (col) {
+        SAR_HIP(hipMemcpyAsync(base + grp_at, col->group_begin.data(), grp_b, hipMemcpyHostToDevice, st));
+        SAR_HIP(hipMemcpyAsync(base + comp_at, col->comps.data(), comp_b, hipMemcpyHostToDevice, st));
+        ColumnDevice d;
+        if ((rc = shape_column_plan(&c, *col, col_rows_first - (uint32_t)lo, d)) != SAR_OK) { (void)hipStreamSynchronize(st); return rc; }
+        d.d_group_begin = (uint32_t*)(base + grp_at); d.d_comps = (sar::ColumnComp*)(base + comp_at);
+        if ((rc = launch_column_plan(&c, d)) != SAR_OK) { (void)hipStreamSynchronize(st); return rc; }
+    }
+    // the result is complete, and the host copies of the tables are no longer needed, when the stream has drained
+    SAR_HIP(hipStreamSynchronize(st));
+    return SAR_OK;
+}
+
+}  // namespace
+
+extern "C" int sar_run_static(int device, void* stream, const sar_schedule* prework, const sar_schedule* main_sched, int n,
+                              void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
+    return guarded([&] { return run_static_body(device, stream, prework, main_sched, n, device_ptrs, bytes_per_rank, dtype); });
+}
+
+extern "C" uint64_t sar_static_scratch_bytes(void) { return SAR_STATIC_SCRATCH_BYTES; }
