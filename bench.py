@@ -9,21 +9,23 @@ before every step, outside the timed region, as the reference re-fills before
 every iteration; each step is timed with HIP events on the executor's stream,
 as the reference times each iteration.
 
-value     = algorithmic bytes of the schedule (16 S) / mean step time
-roofline  = algorithmic bytes per launch / mean launch duration of the dominant
-            kernel (the column kernel: one launch per schedule; with
-            --executor 0 the round kernel: one launch per round), measured live
-            with an event pair around every launch
+value     = bytes that reach memory per step / mean step time: an HBM rate,
+            at most the 8 TB/s peak.  The bytes are the plan's of this very
+            run (sar_stats): the rows' algorithmic bytes (COPY 2, XREDUCE 4,
+            REDUCE_INTO 3 per payload byte) minus the operands the column
+            kernel takes from LDS value slots instead of loading them again
+            and minus the stores it leaves out because they are overwritten
+            unread.  The rocprofv3 counters (profiles/) measure the same
+            number within 0.01 %.
+algorithmic_GBps = the rows' algorithmic bytes / mean step time: every row
+            priced on its own, whether or not its operand came from LDS.  It
+            can pass the HBM peak and is not a roofline fraction.
+roofline  = the same two figures for the dominant kernel (the column kernel:
+            one launch per schedule; with --executor 0 the round kernel: one
+            launch per round) from an event pair around every launch.
+comparators = ring, rhd and direct on the same rank buffers and inputs.
 cpu_baseline = the CPU checker (oracle/, a port) executing the same schedule
-            on the host cores of this box, on a bounded sample
-
-The column executor forwards values: a COPY whose source the same lane wrote in
-an earlier round takes it from an LDS slot instead of loading it again (every
-store still happens).  Those re-reads are part of the algorithmic bytes (each
-row is priced on its own), so `value` can pass what HBM alone could deliver;
-`forwarded_bytes_per_step`, `memory_side_GBps` and `roofline.traffic` say how
-much really went to memory, and `every_operand_loaded` repeats the measurement
-with forwarding switched off (traffic = algorithmic bytes).
+            on the host cores of this box.
 """
 import argparse
 import json
@@ -38,6 +40,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 METRIC = "achieved HBM GB/s (% of roofline) of emulated n-rank AllReduce, 1 MI355X"
+CPU_SHARE = 16      # host threads a one-GPU job may use on the GPU box, whatever the machine's core count
 
 
 def load_table(lib, n):
@@ -50,39 +53,67 @@ def load_table(lib, n):
     return lib.builtin("stragglar", n), "allreduce_%dGPU.cu table" % n
 
 
-def cpu_baseline(lib, ctx, n, elems, table_text_rounds, algorithmic_bytes, budget_s=25.0):
-    """Time the CPU checker on the same workload (inputs downloaded from the device)."""
-    import numpy as np
-    from oracle import load_oracle
-    orc = load_oracle()
-    ctx.restore()
-    inputs = [ctx.download(r) for r in range(n)]
-    out = {}
-    cores = os.cpu_count() or 1
+def host_threads():
+    logical = os.cpu_count() or 1
     try:
-        cores = len(os.sched_getaffinity(0))
+        affinity = len(os.sched_getaffinity(0))
     except Exception:
-        pass
-    cores = min(cores, 16)
-    for label, threads in (("cpu_baseline", 1), ("cpu_baseline_all_cores", cores)):
+        affinity = logical
+    return logical, affinity, max(1, min(affinity, CPU_SHARE))
+
+
+def cpu_run(orc, alg, bufs, rounds):
+    if alg == "stragglar":
+        orc.stragglar(bufs, rounds, "f32")
+    else:
+        orc.run(alg, bufs, "f32", delay=-1.0)
+
+
+def cpu_baseline(orc, inputs, n, elems, rounds, algorithmic_bytes, budget_s=25.0):
+    """Time the CPU checker on the same workload (inputs downloaded from the device)."""
+    out = {}
+    logical, affinity, many = host_threads()
+    bufs = None
+    for label, threads in (("cpu_baseline", 1), ("cpu_baseline_multithread", many)):
         orc.set_threads(threads)
         times = []
         t_begin = time.perf_counter()
         while True:
             bufs = [x.copy() for x in inputs]
             t0 = time.perf_counter()
-            orc.stragglar(bufs, table_text_rounds, "f32")
+            orc.stragglar(bufs, rounds, "f32")
             times.append(time.perf_counter() - t0)
             if len(times) >= 3 or time.perf_counter() - t_begin > budget_s / 2:
                 break
         best = min(times)
         out[label] = {
             "value": round(algorithmic_bytes / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "bytes": "algorithmic (the checker loads every operand)",
+            "host_logical_cpus": logical, "host_cpus_in_affinity_mask": affinity,
             "sample": "%d full pass(es) of the same workload (n=%d, %d fp32 elements per rank), best of %d, %.2f s each"
                       % (len(times), n, elems, len(times), best),
         }
+    out["cpu_baseline_multithread"]["note"] = ("threads = min(CPUs in the affinity mask, %d): a one-GPU job on this pool is granted %d host CPUs "
+                                               "whatever the machine has" % (CPU_SHARE, CPU_SHARE))
     orc.set_threads(1)
     return out, bufs
+
+
+def timed_steps(ctx, steps, warmup):
+    for _ in range(warmup):
+        ctx.restore()
+        ctx.run(-1.0)
+    out = []
+    for _ in range(steps):
+        ctx.restore()                 # untimed: the batch is put back in place, resident in HBM
+        out.append(ctx.run(-1.0))     # start event, the launches, stop event, block on stop
+    return out
+
+
+def rates(st, ms):
+    """(bytes that reach memory per step, HBM GB/s, algorithmic GB/s) for a plan and a step time."""
+    to_memory = st.algorithmic_bytes - st.forwarded_bytes - st.elided_store_bytes
+    return to_memory, to_memory / ms / 1e6, st.algorithmic_bytes / ms / 1e6
 
 
 def main():
@@ -93,7 +124,8 @@ def main():
     ap.add_argument("--ranks", type=int, default=8)
     ap.add_argument("--mib", type=int, default=256, help="unpadded MiB per rank")
     ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and the bit checks against the CPU checker")
+    ap.add_argument("--no-comparators", action="store_true", help="skip ring / rhd / direct on the same buffers")
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
     ap.add_argument("--executor", type=int, default=None, choices=[0, 1, 2],
                     help="0 = one launch per round, 1 = column executor (one launch per schedule), 2 = chosen by the library's cost model (default)")
@@ -127,15 +159,7 @@ def main():
     st = ctx.stats()
     tune = ctx.get_tuning().as_dict()
 
-    for _ in range(args.warmup):
-        ctx.restore()
-        ctx.run(-1.0)
-    step_ms = []
-    t_wall0 = time.perf_counter()
-    for _ in range(args.steps):
-        ctx.restore()                 # untimed: the batch is put back in place, resident in HBM
-        step_ms.append(ctx.run(-1.0)) # start event, the rounds, stop event, block on stop
-    wall_s = time.perf_counter() - t_wall0
+    step_ms = timed_steps(ctx, args.steps, args.warmup)
     identical = ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts)
     ms = statistics.fmean(step_ms)
     # the same K steps back to back on the host clock, no restore in between (the sums just keep growing):
@@ -146,9 +170,9 @@ def main():
         ctx.run(-1.0)
     back_to_back_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ctx.restore()
-    value = st.algorithmic_bytes / ms / 1e6
+    to_memory, hbm_gbps, alg_gbps = rates(st, ms)
 
-    # per-launch durations of the dominant kernel (sar::round_kernel), events on the launch stream
+    # per-launch durations of the dominant kernel, events on the launch stream
     launch_bytes = ctx.launch_bytes()
     per_launch = [0.0] * len(launch_bytes)
     reps = max(3, min(10, args.steps))
@@ -158,10 +182,12 @@ def main():
         for i, t in enumerate(ctx.run_profiled()):
             per_launch[i] += t / reps
     mean_launch_ms = statistics.fmean(per_launch)
-    mean_launch_bytes = statistics.fmean(launch_bytes)
-    achieved = mean_launch_bytes / mean_launch_ms / 1e6
-    traffic = None
-    traffic_table = {}
+    mean_launch_bytes = statistics.fmean(launch_bytes)                      # algorithmic
+    mean_launch_memory = to_memory / len(launch_bytes)                      # what the plan sends to memory
+    achieved = mean_launch_memory / mean_launch_ms / 1e6
+    # What the hardware counters saw of this kernel on this workload, measured offline (two rocprofv3 --pmc runs,
+    # FETCH_SIZE and WRITE_SIZE, calibrated on copy kernels of known size) and kept under profiles/.
+    traffic, traffic_source, traffic_table = None, None, {}
     tpath = os.path.join(ROOT, "profiles", "kernel_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
@@ -169,78 +195,143 @@ def main():
         key = "%s_n%d_%dMiB_f32_%s" % (args.alg, n, args.mib, ("column_forwarding" if st.col_slots else "column") if st.executor == 1 else "rounds")
         if key in traffic_table:
             traffic = traffic_table[key]["hbm_bytes_per_launch"]
+            traffic_source = "offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, %s (not measured by this run)" % traffic_table[key]["source"]
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "bytes": "bytes that reach memory per launch, from this run's plan: algorithmic - taken from LDS slots - stores left out",
+                "memory_bytes_per_launch": int(mean_launch_memory),
+                "traffic": traffic, "traffic_source": traffic_source,
+                "traffic_vs_plan": round(traffic / mean_launch_memory, 4) if traffic and not (st.executor == 1 and not st.col_slots) else None,
                 "kernel": "sar::column_kernel<f32, %d, %s>" % (st.col_block, "forwarding" if st.col_slots else "no forwarding") if st.executor == 1 else "sar::round_kernel<f32, %d, %d>" % (tune["unroll"], tune["block"]),
-                "launches": len(launch_bytes),
-                "algorithmic_bytes_per_launch": int(mean_launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5)}
-    kept_on_chip = st.forwarded_bytes + st.elided_store_bytes
-    if kept_on_chip:
-        roofline["note"] = ("frac can pass 1: %.1f %% of the algorithmic bytes are re-reads of values the same lane wrote, served from LDS%s; "
-                            "the memory side (traffic) ran at %.0f GB/s" % (100.0 * st.forwarded_bytes / st.algorithmic_bytes,
-                                                                          ", and %.1f %% are stores of partial sums that are overwritten unread and left out" % (100.0 * st.elided_store_bytes / st.algorithmic_bytes) if st.elided_store_bytes else "",
-                                                                          (mean_launch_bytes - kept_on_chip / len(launch_bytes)) / mean_launch_ms / 1e6))
-    # the reduce steps alone: the XREDUCE share of every launch is 4 chunk-bytes
+                "launches": len(launch_bytes), "mean_launch_ms": round(mean_launch_ms, 5),
+                "algorithmic_bytes_per_launch": int(mean_launch_bytes),
+                "algorithmic_GBps": round(mean_launch_bytes / mean_launch_ms / 1e6, 1),
+                "algorithmic_frac": round(mean_launch_bytes / mean_launch_ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    if st.executor == 1 and not st.col_slots:
+        roofline["note"] = ("with every operand loaded the plan's bytes equal the algorithmic bytes, but re-reads of a work item hit the XCD's own L2: "
+                            "the counters (traffic) are the HBM-side figure here")
+    logical, affinity, many = host_threads()
     rec = {
-        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "metric": METRIC, "value": round(hbm_gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: n=%d %s (%s), %d MiB fp32 per rank padded to %d B, uniform[-1,1) seeded per rank, "
-                               "DELAY=-1, %d ranks resident in one GPU's HBM" % (n, args.alg, table_name, args.mib, nbytes, n),
+                               "DELAY=-1, %d ranks resident in one GPU's HBM; value = bytes that reach memory per step / step time "
+                               "(an HBM rate; the rows' algorithmic bytes / step time is algorithmic_GBps)" % (n, args.alg, table_name, args.mib, nbytes, n),
                    "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph), "tuning": tune, "executor_used": "column" if st.executor == 1 else "rounds"},
-        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
+        "memory_bytes_per_step": int(to_memory),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
+        "algorithmic_GBps": round(alg_gbps, 1),
+        "algorithmic_frac": round(alg_gbps / HBM_PEAK_GBPS, 4),
         # part of the algorithmic bytes that never leaves the compute unit: re-reads of values the same lane wrote
         # in an earlier round, taken from LDS slots
         "forwarded_bytes_per_step": int(st.forwarded_bytes),
         # stores of values that a later row overwrites before anybody loads them (none in the StragglAR tables)
         "elided_store_bytes_per_step": int(st.elided_store_bytes),
-        "memory_side_GBps": round((st.algorithmic_bytes - st.forwarded_bytes - st.elided_store_bytes) / ms / 1e6, 1),
-        "ms_per_step_min": round(min(step_ms), 5), "wall_ms_per_step_incl_restore": round(wall_s * 1e3 / args.steps, 4),
+        "ms_per_step_min": round(min(step_ms), 5),
         "wall_ms_per_step_back_to_back": round(back_to_back_ms, 4),
         "ranks_identical_after_run": bool(identical),
         # 1 = the two halves of the rank buffers were placed in different regions of HBM (sar_alloc_ranks)
         "arena_spread": int(st.arena_spread),
+        "host": {"logical_cpus": logical, "cpus_in_affinity_mask": affinity, "threads_used_by_multithread_legs": many},
         "roofline": roofline,
     }
     if st.col_slots and args.forward is None:
-        # the same steps with every operand loaded from the rank buffers (traffic = algorithmic bytes)
+        # the same steps with every operand loaded from the rank buffers
         ctx.set_tuning(col_forward=0)
         ctx.prepare(main_sched, None, use_graph=args.graph)
-        plain_ms = []
-        for i in range(args.warmup + args.steps):
-            ctx.restore()
-            t = ctx.run(-1.0)
-            if i >= args.warmup:
-                plain_ms.append(t)
+        plain_ms = timed_steps(ctx, args.steps, args.warmup)
         pm = statistics.fmean(plain_ms)
-        rec["every_operand_loaded"] = {"value": round(st.algorithmic_bytes / pm / 1e6, 1), "unit": "GB/s", "ms_per_step": round(pm, 5),
-                                       "frac_of_hbm_peak": round(st.algorithmic_bytes / pm / 1e6 / HBM_PEAK_GBPS, 4),
-                                       "ranks_identical_after_run": bool(ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts))}
+        leg = {"algorithmic_GBps": round(st.algorithmic_bytes / pm / 1e6, 1), "unit": "GB/s", "ms_per_step": round(pm, 5),
+               "algorithmic_frac": round(st.algorithmic_bytes / pm / 1e6 / HBM_PEAK_GBPS, 4),
+               "ranks_identical_after_run": bool(ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts)),
+               "note": "not an HBM rate: re-reads of a work item hit the XCD's own L2"}
         plain_key = "%s_n%d_%dMiB_f32_column" % (args.alg, n, args.mib)
         if plain_key in traffic_table:
             # what the counters saw of it: re-reads of an item that hit the XCD's own L2 never reach the fabric
-            rec["every_operand_loaded"]["traffic"] = traffic_table[plain_key]["hbm_bytes_per_launch"]
-            rec["every_operand_loaded"]["memory_side_GBps"] = round(traffic_table[plain_key]["hbm_bytes_per_launch"] / pm / 1e6, 1)
+            leg["traffic"] = traffic_table[plain_key]["hbm_bytes_per_launch"]
+            leg["traffic_source"] = "offline rocprofv3 --pmc, %s" % traffic_table[plain_key]["source"]
+            leg["memory_side_GBps"] = round(traffic_table[plain_key]["hbm_bytes_per_launch"] / pm / 1e6, 1)
+            leg["frac_of_hbm_peak"] = round(leg["memory_side_GBps"] / HBM_PEAK_GBPS, 4)
+        rec["every_operand_loaded"] = leg
         ctx.set_tuning(col_forward=1)
         ctx.prepare(main_sched, None, use_graph=False)
+
+    if args.alg == "stragglar" and st.col_slots and 2 <= n - 1 <= 8:
+        # What the memory system delivers for this kernel's own mix of streams, by a kernel that does nothing else
+        # (sar_probe_streams, fastest of 72 launch shapes): per chunk index r the cold reads of rank r's and the
+        # straggler's chunk r and the stores of their sum to every rank, on the same buffers in the same places.
+        chunk = (elems // (n - 1)) * 4
+        res = ctx.probe_streams([([r, n - 1], list(range(n)), r * chunk) for r in range(n - 1)], chunk - chunk % 16, 5)
+        rec["stream_ceiling"] = {"mix": "%d x (2 streams read + %d written), %d B each: the schedule's traffic once re-reads come from LDS" % (n - 1, n, chunk - chunk % 16),
+                                 "GBps": round(res.gbps, 1), "frac_of_hbm_peak": round(res.gbps / HBM_PEAK_GBPS, 4), "ms": round(res.best_ms, 5),
+                                 "shape": {"block": res.block, "vectors_per_thread": res.unroll, "streaming": res.nontemporal, "resident_grid": res.persistent, "jobs_take_turns": res.interleave},
+                                 "shapes_tried": res.variants, "slowest_shape_ms": round(res.worst_ms, 5),
+                                 "kernel_vs_ceiling": round(roofline["achieved"] / res.gbps, 4)}
+        ctx.restore()
+
+    orc = inputs = None
+    if not args.no_cpu:
+        import numpy as np
+        from oracle import load_oracle, parse_table
+        orc = load_oracle()
+        ctx.restore()
+        inputs = [ctx.download(r) for r in range(n)]
+
+    def bit_exact(alg, rounds):
+        """The GPU result of one step against the CPU checker's, bit for bit, at the full size."""
+        orc.set_threads(many)
+        want = [x.copy() for x in inputs]
+        cpu_run(orc, alg, want, rounds)
+        orc.set_threads(1)
+        ctx.restore()
+        ctx.run(-1.0)
+        return all(np.array_equal(ctx.download(r).view(np.uint32), want[r].view(np.uint32)) for r in range(n))
+
     if not args.no_cpu and args.alg == "stragglar":
-        from oracle import parse_table
         gold = os.path.join(ROOT, "tests", "golden", "stragglar_n%d_cu.txt" % n)
         path = os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)
         with open(path if os.path.exists(path) else gold) as f:
             rounds = parse_table(f.read())
-        base, cpu_out = cpu_baseline(lib, ctx, n, elems, rounds, st.algorithmic_bytes)
+        base, cpu_out = cpu_baseline(orc, inputs, n, elems, rounds, st.algorithmic_bytes)
         rec.update(base)
-        # the timed GPU result against the checker's, bit for bit, at the full size
-        import numpy as np
         ctx.restore()
         ctx.run(-1.0)
         ok = all(np.array_equal(ctx.download(r).view(np.uint32), cpu_out[r].view(np.uint32)) for r in range(n))
         rec["bit_exact_vs_cpu_checker"] = bool(ok)
+
+    if not args.no_comparators and args.alg == "stragglar":
+        # configs[1]: "ring, rhd and direct schedules run on the same buffers for comparison"
+        # (allreduce_8GPU.cu:146-198, :221-532, :60-113): same rank buffers, same inputs, same step protocol
+        comps = {}
+        for alg in ("ring", "rhd", "direct"):
+            if alg == "rhd" and n & (n - 1):
+                continue
+            if alg == "direct" and n % 2:
+                continue
+            sched = lib.builtin(alg, n)
+            ctx.prepare(sched, None, use_graph=args.graph)
+            cst = ctx.stats()
+            cms = timed_steps(ctx, args.steps, args.warmup)
+            cm = statistics.fmean(cms)
+            cmem, chbm, calg = rates(cst, cm)
+            leg = {"ms_per_step": round(cm, 5), "ms_per_step_min": round(min(cms), 5),
+                   "memory_side_GBps": round(chbm, 1), "frac_of_hbm_peak": round(chbm / HBM_PEAK_GBPS, 4),
+                   "memory_bytes_per_step": int(cmem), "algorithmic_bytes_per_step": int(cst.algorithmic_bytes),
+                   "algorithmic_GBps": round(calg, 1), "executor_used": "column" if cst.executor == 1 else "rounds",
+                   "launches": int(cst.launches),
+                   "ranks_identical_after_run": bool(ctx.ranks_identical((elems // sched.parts) * sched.parts))}
+            if orc is not None:
+                leg["bit_exact_vs_cpu_checker"] = bool(bit_exact(alg, None))
+            comps[alg] = leg
+        rec["comparators"] = comps
     ctx.close()
     print(json.dumps(rec))
-    if not identical or rec.get("bit_exact_vs_cpu_checker") is False:
+    bad = not identical or rec.get("bit_exact_vs_cpu_checker") is False
+    for leg in rec.get("comparators", {}).values():
+        bad = bad or not leg["ranks_identical_after_run"] or leg.get("bit_exact_vs_cpu_checker") is False
+    if bad:
         sys.exit(1)
 
 

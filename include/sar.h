@@ -107,7 +107,8 @@ typedef struct sar_tuning_t {
                           /*     main schedule, each workgroup walking all rounds for its own range  */
                           /*     of within-chunk offsets (schedules with MREDUCE rows fall back to   */
                           /*     0); 2 = whichever a small cost model expects to be faster (default) */
-    int32_t col_wgs;      /* column executor: workgroups per compute unit in the grid                */
+    int32_t col_wgs;      /* column executor: most workgroups per compute unit in the grid (they stride over */
+                          /*     the work items); 0 = chosen by the library (default)                       */
     int32_t col_block;    /* column executor: threads per workgroup = 16-byte vectors per column     */
                           /*     (256, 512 or 1024; 0 = chosen from the number of columns)           */
     int32_t col_forward;  /* column executor: 1 = a value a lane wrote in an earlier round and needs  */
@@ -148,6 +149,11 @@ typedef struct sar_tuning_t {
                           /*     buffers in different thirds of the 288 GiB disturb each other less; */
                           /*     the pair is kept for the life of the context); ranks back to back  */
                           /*     when no such pair is found or the device lacks the room; 0 = never  */
+    int32_t col_prework;  /* 1 = multi-source rows run in the column kernel as well: the pre-work that      */
+                          /*     overlaps the straggler's delay is one column launch on the second stream,  */
+                          /*     and so is a schedule that consists of such rows (the pre-work timed on its */
+                          /*     own); 0 = they run in the multi-source kernel, one launch per round.       */
+                          /*     Rows that are not whole 16-byte vectors on vector boundaries always do     */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */
@@ -309,6 +315,28 @@ int sar_run_profiled(sar_ctx* ctx, float* ms, int cap, int* count);
  * order (the denominator-free half of a per-kernel roofline figure). */
 int sar_launch_bytes(sar_ctx* ctx, uint64_t* bytes, int cap, int* count);
 
+/* What the memory system delivers for a mix of read and written streams laid over the rank buffers where they
+ * are: the yardstick for the data kernels (no counterpart in the reference, which is bound by its links).  A job
+ * is nread streams read and nwrite streams written, each `bytes` long, starting byte_off into the named ranks'
+ * buffers; every 16-byte vector written is the fp32 sum of the job's read streams.  A rank named on both sides is
+ * updated in place, as the two sides of an exchange are (allreduce_8GPU.cu:564-578 followed by reduce_add :29-34).
+ * All jobs of a call run in one launch of a kernel that does nothing else, in 36 (one job) or 72 shapes --
+ * 256/512/1024 threads x 1/2/4 vectors per thread x cached/streaming accesses x one tile per workgroup or a
+ * resident grid x jobs one after the other or taking turns --, each timed `reps` times with events after one
+ * warm-up launch; the result names the fastest shape.  THE RANK BUFFERS ARE OVERWRITTEN. */
+typedef struct sar_probe_job {
+    int32_t nread, nwrite;            /* 0..8 each, not both 0; all jobs of a call have the same nread */
+    int32_t read_rank[8], write_rank[8];
+    uint64_t byte_off;                /* into each named rank buffer; the streams must start on 16-byte boundaries */
+} sar_probe_job;
+typedef struct sar_probe_result {
+    float best_ms, worst_ms;          /* fastest and slowest shape (each the minimum over its reps) */
+    int32_t block, unroll, nontemporal, persistent, interleave;      /* the fastest shape */
+    int32_t variants;                 /* shapes tried */
+    uint64_t bytes_moved;             /* (nread + nwrite) * bytes summed over the jobs */
+} sar_probe_result;
+int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out);
+
 /* Ticks of the device's constant-rate wall clock that delay_ms lasts: the
  * figure the CLI prints as "Sleep cycles" (calculate_sleep_cycles,
  * allreduce_8GPU.cu:47-58, uses ms * clockRate_kHz of the shader clock). */
@@ -357,8 +385,9 @@ typedef struct sar_plan_row {
 
 typedef struct sar_plan_ptr { int32_t rank; int32_t reserved; uint64_t off; } sar_plan_ptr;
 
-/* The rows behind sar_plan(): the column executor's plan for the main schedule (same_launch 0) or for pre-work
- * and main schedule in one launch (same_launch 1), whether or not the cost model would pick that executor.
+/* The rows behind sar_plan(): the column executor's plan for the main schedule (same_launch 0), for pre-work
+ * and main schedule in one launch (same_launch 1) or for the pre-work alone (same_launch 2), whether or not
+ * the cost model would pick that executor.
  * Writes at most row_cap rows and ptr_cap pointer-list entries; *nrows and *nptrs are the full counts.
  * SAR_ESTATE when there is no such plan (executor 0, rows the column kernel cannot run, no pre-work).
  * Host only; for tools and for tests that check the plan row by row. */

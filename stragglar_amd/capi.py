@@ -58,9 +58,24 @@ class PlanPtr(ctypes.Structure):
     _fields_ = [("rank", ctypes.c_int32), ("reserved", ctypes.c_int32), ("off", ctypes.c_uint64)]
 
 
+class ProbeJob(ctypes.Structure):
+    _fields_ = [("nread", ctypes.c_int32), ("nwrite", ctypes.c_int32), ("read_rank", ctypes.c_int32 * 8),
+                ("write_rank", ctypes.c_int32 * 8), ("byte_off", ctypes.c_uint64)]
+
+
+class ProbeResult(ctypes.Structure):
+    _fields_ = [("best_ms", ctypes.c_float), ("worst_ms", ctypes.c_float), ("block", ctypes.c_int32), ("unroll", ctypes.c_int32),
+                ("nontemporal", ctypes.c_int32), ("persistent", ctypes.c_int32), ("interleave", ctypes.c_int32),
+                ("variants", ctypes.c_int32), ("bytes_moved", ctypes.c_uint64)]
+
+    @property
+    def gbps(self) -> float:
+        return self.bytes_moved / self.best_ms / 1e6
+
+
 class Tuning(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd", "segments",
-                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "col_fuse_copies", "arena_spread")]
+                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "col_fuse_copies", "arena_spread", "col_prework")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -85,7 +100,7 @@ EXPORTS = [
     "sar_fill_reference_pattern", "sar_fill_uniform", "sar_fill_normal", "sar_snapshot", "sar_restore",
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
-    "sar_run_static", "sar_static_scratch_bytes", "sar_rank_pointer",
+    "sar_run_static", "sar_static_scratch_bytes", "sar_rank_pointer", "sar_probe_streams",
 ]
 
 
@@ -143,6 +158,7 @@ class Library:
             "sar_run_static": (c_int, [c_int, vp, vp, vp, c_int, P(vp), u64, c_int]),
             "sar_static_scratch_bytes": (u64, []),
             "sar_rank_pointer": (c_int, [vp, c_int, P(vp)]),
+            "sar_probe_streams": (c_int, [vp, c_int, P(ProbeJob), u64, c_int, P(ProbeResult)]),
         }
         assert sorted(sig) == sorted(EXPORTS)
         for name, (res, args) in sig.items():
@@ -393,6 +409,20 @@ class Context:
         cnt = ctypes.c_int(0)
         self._c(self._lib.lib.sar_launch_bytes(self._h, buf, cap, ctypes.byref(cnt)))
         return [int(buf[i]) for i in range(min(cap, cnt.value))]
+
+    def probe_streams(self, jobs, nbytes: int, reps: int = 5) -> ProbeResult:
+        """The memory system's rate for a mix of streams over the rank buffers (which are overwritten).
+        ``jobs``: a list of (read_ranks, write_ranks, byte_off)."""
+        arr = (ProbeJob * len(jobs))()
+        for j, (rd, wr, off) in enumerate(jobs):
+            arr[j].nread, arr[j].nwrite, arr[j].byte_off = len(rd), len(wr), off
+            for k, r in enumerate(rd):
+                arr[j].read_rank[k] = r
+            for k, r in enumerate(wr):
+                arr[j].write_rank[k] = r
+        res = ProbeResult()
+        self._c(self._lib.lib.sar_probe_streams(self._h, len(jobs), arr, nbytes, reps, ctypes.byref(res)))
+        return res
 
     def sleep_ticks(self, delay_ms: float) -> int:
         t = ctypes.c_int64(0)

@@ -93,7 +93,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 64, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 0, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -108,6 +108,7 @@ struct sar_ctx {
     bool column = false;
     ColumnDevice col;                  // the main schedule
     ColumnDevice fused;                // pre-work + main schedule in one launch (used by sar_run with no delay)
+    ColumnDevice pre;                  // the pre-work alone as one column launch (runs beside the straggler's delay)
     int cu_count = 0;
 
     std::vector<char*> adopted;        // caller-owned rank buffers (sar_adopt_ranks); empty when the arena is in use
@@ -131,7 +132,7 @@ void drop_plan(sar_ctx* c) {
     if (c->graph_fused) { (void)hipGraphDestroy(c->graph_fused); c->graph_fused = nullptr; }
     if (c->d_ops) { (void)hipFree(c->d_ops); c->d_ops = nullptr; }
     if (c->d_ptrs) { (void)hipFree(c->d_ptrs); c->d_ptrs = nullptr; }
-    for (ColumnDevice* d : {&c->col, &c->fused}) {
+    for (ColumnDevice* d : {&c->col, &c->fused, &c->pre}) {
         if (d->d_group_begin) (void)hipFree(d->d_group_begin);
         if (d->d_comps) (void)hipFree(d->d_comps);
         *d = ColumnDevice{};
@@ -448,16 +449,17 @@ bool column_pays(const sar_ctx* c, const ColumnPlan& cp) {
     return est_column <= est_rounds;
 }
 
-int launch_column_plan(sar_ctx* c, const ColumnDevice& d) {
+int launch_column_plan(sar_ctx* c, const ColumnDevice& d, hipStream_t st) {
     sar::ColumnLaunch L{};
     L.ops = c->d_ops + d.first_op; L.group_begin = d.d_group_begin; L.comps = d.d_comps; L.ptrs = c->d_ptrs;
     L.ncomp = d.ncomp; L.nitems = d.items;
     L.table_rows = d.table_rows; L.table_groups = d.table_groups;
     L.lane_local = d.lane_local; L.policy = d.policy; L.multi_source = d.multi_source;
     L.ncols = d.ncols; L.run = d.run;
-    SAR_HIP(sar::launch_column(c->dtype, (int)d.block, d.grid, d.slots, c->stream, L));
+    SAR_HIP(sar::launch_column(c->dtype, (int)d.block, d.grid, d.slots, st, L));
     return SAR_OK;
 }
+int launch_column_plan(sar_ctx* c, const ColumnDevice& d) { return launch_column_plan(c, d, c->stream); }
 
 // Launch shape of a column plan whose rows sit in the row table from `first_op` on (no device work).
 int shape_column_plan(const sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, ColumnDevice& d) {
@@ -475,8 +477,12 @@ int shape_column_plan(const sar_ctx* c, const ColumnPlan& cp, uint32_t first_op,
     d.first_op = first_op; d.ncomp = (uint32_t)cp.comps.size(); d.ncols = (uint32_t)ncols;
     d.run = cp.component_major ? (uint32_t)ncols : 1u;        // d.run divides ncols either way: no padding items
     d.items = (uint32_t)items;
-    const uint64_t resident = (uint64_t)std::max(1, c->cu_count) * (uint64_t)std::max(1, c->tune.col_wgs);
-    d.grid = (uint32_t)std::min<uint64_t>(items, resident);
+    // Grid: one workgroup per item, so that the workgroups resident at a time work on neighbouring items (a smaller
+    // grid whose workgroups stride over the items has them on several distant ranges at once: n = 8, 1 GiB per
+    // rank, 2 to 4 % slower for all four algorithms).  A launch of multi-source rows alone is the exception: seven
+    // reads per vector run 2 % faster from 64 workgroups per compute unit striding.
+    const uint64_t per_cu = c->tune.col_wgs > 0 ? (uint64_t)c->tune.col_wgs : (cp.multi_source && cp.nslots == 0 ? 64u : 4096u);
+    d.grid = (uint32_t)std::min<uint64_t>(items, (uint64_t)std::max(1, c->cu_count) * per_cu);
     return SAR_OK;
 }
 
@@ -511,29 +517,39 @@ int launch_all(sar_ctx* c, const std::vector<Launch>& v) { return launch_all(c, 
 
 int launch_main(sar_ctx* c) { return c->column ? launch_column_plan(c, c->col) : launch_all(c, c->rounds); }
 
+// The column plans sar_prepare may use, and whether it does.
+struct HostPlans {
+    ColumnPlan cp, fp, pp;             // the main schedule; pre-work + main schedule in one launch; the pre-work alone
+    uint32_t col_first = 0, fused_first = 0, pre_first = 0;      // their first rows in the row table
+    bool want_column = false, want_fused = false, want_pre = false;
+};
+
 // Everything sar_prepare decides, on the host alone: the rows of both executors, and whether the column executor runs.
 int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, std::vector<sar::DevOp>& rows,
-                 std::vector<char*>& ptrs, ColumnPlan& cp, uint32_t* col_first, bool* want_column,
-                 ColumnPlan& fused, uint32_t* fused_first, bool* want_fused) {
+                 std::vector<char*>& ptrs, HostPlans& hp) {
     int rc;
-    *col_first = 0; *want_column = false; *fused_first = 0; *want_fused = false;
+    hp = HostPlans();
     try {
         if (prework && (rc = lower(c, prework->s, rows, ptrs, c->prework, &main_sched->s)) != SAR_OK) return rc;
         if ((rc = lower(c, main_sched->s, rows, ptrs, c->rounds, nullptr)) != SAR_OK) return rc;
         sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &c->stats.algorithmic_bytes, nullptr);
         bool columnar = c->tune.executor != 0;
-        for (const auto& L : c->rounds) if (L.mreduce) columnar = false;     // multi-source rows run one launch per round
+        bool multi_source = false;
+        for (const auto& L : c->rounds) multi_source |= L.mreduce;
+        // a schedule of multi-source rows (the pre-work timed on its own) runs as column launches when col_prework says so
+        if (multi_source && !c->tune.col_prework) columnar = false;
         if (columnar) {
-            *col_first = (uint32_t)rows.size();
-            if ((rc = lower_column(c, {&main_sched->s}, rows, ptrs, cp)) != SAR_OK) return rc;
-            columnar = rows.size() > *col_first && !cp.unsupported;
+            hp.col_first = (uint32_t)rows.size();
+            if ((rc = lower_column(c, {&main_sched->s}, rows, ptrs, hp.cp)) != SAR_OK) return rc;
+            columnar = rows.size() > hp.col_first && !hp.cp.unsupported;
         }
-        if (columnar && c->tune.executor == 2) columnar = column_pays(c, cp);
-        *want_column = columnar;
+        // (multi-source rows: measured, the column kernel is the faster one at every size, see mreduce_kernel)
+        if (columnar && c->tune.executor == 2 && !multi_source) columnar = column_pays(c, hp.cp);
+        hp.want_column = columnar;
         // Pre-work and main schedule as ONE launch, for runs in which nobody is late (the pre-work then simply
         // precedes the schedule): its result for a chunk is handed to the exchange of that chunk in a value slot.
         if (columnar && prework && c->tune.col_fuse_prework) {
-            *fused_first = (uint32_t)rows.size();
+            hp.fused_first = (uint32_t)rows.size();
             // A schedule of whole-buffer rows (direct) behind a pre-work that is cut into chunks: the same rows,
             // written over the pre-work's chunks (the last one takes the elements past the last chunk boundary
             // along, as the pre-work's last row does).
@@ -550,14 +566,21 @@ int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* ma
                     }
                 if (whole) second = &recut;
             }
-            if ((rc = lower_column(c, {&prework->s, second}, rows, ptrs, fused)) != SAR_OK) return rc;
-            *want_fused = rows.size() > *fused_first && !fused.unsupported;
+            if ((rc = lower_column(c, {&prework->s, second}, rows, ptrs, hp.fp)) != SAR_OK) return rc;
+            hp.want_fused = rows.size() > hp.fused_first && !hp.fp.unsupported;
+        }
+        // The pre-work alone as one column launch, for runs in which it overlaps the straggler's delay (and for
+        // runs without a delay when there is no single launch for both).
+        if (prework && c->tune.executor != 0 && c->tune.col_prework) {
+            hp.pre_first = (uint32_t)rows.size();
+            if ((rc = lower_column(c, {&prework->s}, rows, ptrs, hp.pp)) != SAR_OK) return rc;
+            hp.want_pre = rows.size() > hp.pre_first && !hp.pp.unsupported;
         }
     } catch (const std::bad_alloc&) { return set_error(SAR_ENOMEM, "out of host memory"); }
     return SAR_OK;
 }
 
-sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column, bool fused) {
+sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column, bool fused, bool pre_column) {
     sar_stats_t st{};
     sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
     if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
@@ -565,7 +588,8 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     for (const auto& r : main_sched->s.rounds) st.ops += (int)r.size();
     if (column) st.launches += 1;
     else for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
-    for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
+    if (pre_column) st.launches += 1;
+    else for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
     st.executor = column ? 1 : 0;
     st.col_block = column ? (int32_t)cp.block : 0;
     st.col_slots = column ? (int32_t)cp.nslots : 0;
@@ -581,13 +605,13 @@ bool valid_tuning(const sar_tuning_t& t) {
     return (t.block == 256 || t.block == 512) && (t.unroll == 1 || t.unroll == 2 || t.unroll == 4 || t.unroll == 8) &&
            (t.order == 0 || t.order == 1) && t.cache_policy >= 0 && t.cache_policy <= 3 && t.reuse_rounds >= 0 && t.reuse_rounds <= 64 &&
            (t.reverse_odd == 0 || t.reverse_odd == 1) && t.segments >= 0 && t.segments <= 256 &&
-           (t.executor >= 0 && t.executor <= 2) && t.col_wgs >= 1 && t.col_wgs <= 4096 &&
+           (t.executor >= 0 && t.executor <= 2) && t.col_wgs >= 0 && t.col_wgs <= 4096 &&
            (t.col_block == 0 || t.col_block == 256 || t.col_block == 512 || t.col_block == 1024) &&
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
            (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1) && t.col_fuse_copies >= 0 && t.col_fuse_copies <= 2 &&
-           (t.arena_spread == 0 || t.arena_spread == 1);
+           (t.arena_spread == 0 || t.arena_spread == 1) && (t.col_prework == 0 || t.col_prework == 1);
 }
 
 // sar_plan / sar_plan_rows: a context that never touches the device, with the rank buffers at made-up, suitably
@@ -596,9 +620,7 @@ struct HostPlan {
     sar_ctx c;
     uint64_t stride = 0;
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    ColumnPlan cp, fp;
-    uint32_t col_first = 0, fused_first = 0;
-    bool want_column = false, want_fused = false;
+    HostPlans hp;
 
     int make(const sar_schedule* prework, const sar_schedule* main_sched, int n, uint64_t bytes_per_rank, int dtype,
              const sar_tuning_t* tuning, int compute_units) {
@@ -619,7 +641,7 @@ struct HostPlan {
         if (tuning) c.tune = *tuning;
         stride = (bytes_per_rank + (2u << 20) - 1) & ~(uint64_t)((2u << 20) - 1);
         for (int r = 0; r < n; ++r) c.adopted.push_back(reinterpret_cast<char*>((uintptr_t)1 << 40) + (uint64_t)r * stride);
-        return plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused);
+        return plan_on_host(&c, prework, main_sched, rows, ptrs, hp);
     }
 };
 
@@ -1003,8 +1025,8 @@ static int prepare_body(sar_ctx* c, const sar_schedule* prework, const sar_sched
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_plan(c);
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    ColumnPlan cp, fp; uint32_t col_first = 0, fused_first = 0; bool want_column = false, want_fused = false;
-    int rc = plan_on_host(c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused);
+    HostPlans hp;
+    int rc = plan_on_host(c, prework, main_sched, rows, ptrs, hp);
     if (rc != SAR_OK) { drop_plan(c); return rc; }
     if (!rows.empty()) {
         SAR_HIP(hipMalloc((void**)&c->d_ops, rows.size() * sizeof(sar::DevOp)));
@@ -1013,13 +1035,14 @@ static int prepare_body(sar_ctx* c, const sar_schedule* prework, const sar_sched
     SAR_HIP(hipMalloc((void**)&c->d_ptrs, (ptrs.size() + 1) * sizeof(char*)));
     if (!ptrs.empty()) SAR_HIP(hipMemcpy(c->d_ptrs, ptrs.data(), ptrs.size() * sizeof(char*), hipMemcpyHostToDevice));
 
-    if (want_column) {
-        if ((rc = upload_column_plan(c, cp, col_first, c->col)) != SAR_OK) { drop_plan(c); return rc; }
+    if (hp.want_column) {
+        if ((rc = upload_column_plan(c, hp.cp, hp.col_first, c->col)) != SAR_OK) { drop_plan(c); return rc; }
         c->column = true;
-        if (want_fused && (rc = upload_column_plan(c, fp, fused_first, c->fused)) != SAR_OK) { drop_plan(c); return rc; }
+        if (hp.want_fused && (rc = upload_column_plan(c, hp.fp, hp.fused_first, c->fused)) != SAR_OK) { drop_plan(c); return rc; }
     }
+    if (hp.want_pre && (rc = upload_column_plan(c, hp.pp, hp.pre_first, c->pre)) != SAR_OK) { drop_plan(c); return rc; }
 
-    sar_stats_t st = plan_stats(c, prework, main_sched, cp, c->column, c->fused.ready);
+    sar_stats_t st = plan_stats(c, prework, main_sched, hp.cp, c->column, c->fused.ready, c->pre.ready);
     if (use_graph) {
         // the main rounds as one graph, and the single launch of pre-work + schedule (what sar_run with delay 0
         // runs) as another: kernel nodes only (no memset nodes)
@@ -1059,7 +1082,7 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
         main_done = true;
     } else if (delay_ms == 0) {
         // nobody is late: pre-work, then the schedule, on one stream
-        int rc = launch_all(c, c->prework); if (rc) return rc;
+        int rc = c->pre.ready ? launch_column_plan(c, c->pre) : launch_all(c, c->prework); if (rc) return rc;
     } else if (delay_ms > 0) {
         // The straggler is busy for delay_ms (gpu_sleep_kernel on its stream, allreduce_8GPU.cu:876-889) while the
         // others do their pre-work.  Here the wait sits on the stream that goes on to run the schedule and the
@@ -1068,7 +1091,7 @@ int sar_run(sar_ctx* c, float delay_ms, float* elapsed_ms) {
         // straggler's arrival than with the join of the two streams on the critical path).
         const uint64_t ticks = (uint64_t)((double)delay_ms * (double)c->wall_khz);
         SAR_HIP(hipStreamWaitEvent(c->prework_stream, c->ev_start, 0));
-        int rc = launch_all(c, c->prework, c->prework_stream); if (rc) return rc;
+        int rc = c->pre.ready ? launch_column_plan(c, c->pre, c->prework_stream) : launch_all(c, c->prework, c->prework_stream); if (rc) return rc;
         SAR_HIP(hipEventRecord(c->ev_join, c->prework_stream));
         SAR_HIP(sar::launch_sleep(c->stream, ticks));
         SAR_HIP(hipStreamWaitEvent(c->stream, c->ev_join, 0));
@@ -1137,6 +1160,61 @@ int sar_launch_bytes(sar_ctx* c, uint64_t* bytes, int cap, int* count) {
     return SAR_OK;
 }
 
+static int probe_streams_body(sar_ctx* c, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out) {
+    if (!c || !c->has_ranks()) return set_error(SAR_ESTATE, "no rank buffers allocated");
+    if (!jobs || !out || njobs < 1 || njobs > 8 || reps < 1 || reps > 1000) return set_error(SAR_EINVAL, "bad argument");
+    if (bytes < 16 || (bytes & 15u)) return set_error(SAR_EINVAL, "bytes must be a positive multiple of 16");
+    sar::ProbeJobs J{};
+    J.njobs = (uint32_t)njobs; J.bytes = bytes;
+    uint64_t moved = 0;
+    for (int j = 0; j < njobs; ++j) {
+        const sar_probe_job& b = jobs[j];
+        if (b.nread < 0 || b.nread > 8 || b.nwrite < 0 || b.nwrite > 8 || b.nread + b.nwrite == 0 || b.nread != jobs[0].nread)
+            return set_error(SAR_EINVAL, "a job has 0 to 8 read and 0 to 8 written streams, and all jobs read equally many");
+        if (b.byte_off > c->bytes_per_rank || bytes > c->bytes_per_rank - b.byte_off) return set_error(SAR_EINVAL, "a job leaves the rank buffer");
+        J.nread[j] = (uint32_t)b.nread; J.nwrite[j] = (uint32_t)b.nwrite;
+        for (int k = 0; k < b.nread + b.nwrite; ++k) {
+            const int rank = k < b.nread ? b.read_rank[k] : b.write_rank[k - b.nread];
+            if (rank < 0 || rank >= c->n) return set_error(SAR_EINVAL, "rank out of range");
+            char* p = c->rank_base(rank) + b.byte_off;
+            if ((uintptr_t)p & 15u) return set_error(SAR_EINVAL, "a stream does not start on a 16-byte boundary");
+            if (k < b.nread) J.rd[j][k] = p; else J.wr[j][k - b.nread] = p;
+        }
+        moved += (uint64_t)(b.nread + b.nwrite) * bytes;
+    }
+    SAR_HIP(hipSetDevice(c->device));
+    while (c->ev_prof.size() < 2) { hipEvent_t e; SAR_HIP(hipEventCreate(&e)); c->ev_prof.push_back(e); }
+    *out = sar_probe_result{};
+    out->bytes_moved = moved;
+    for (int block : {256, 512, 1024})
+        for (int unroll : {1, 2, 4})
+            for (int nt = 0; nt < 2; ++nt)
+                for (int persistent = 0; persistent < 2; ++persistent)
+                    for (int interleave = 0; interleave < (njobs > 1 ? 2 : 1); ++interleave) {
+                        float best = -1.f;
+                        for (int r = 0; r <= reps; ++r) {                   // the first run warms up and is not counted
+                            SAR_HIP(hipEventRecord(c->ev_prof[0], c->stream));
+                            SAR_HIP(sar::launch_stream_probe(c->stream, J, block, unroll, nt != 0, persistent != 0, interleave != 0, c->cu_count));
+                            SAR_HIP(hipEventRecord(c->ev_prof[1], c->stream));
+                            SAR_HIP(hipEventSynchronize(c->ev_prof[1]));
+                            float ms = 0.f;
+                            SAR_HIP(hipEventElapsedTime(&ms, c->ev_prof[0], c->ev_prof[1]));
+                            if (r > 0 && (best < 0.f || ms < best)) best = ms;
+                        }
+                        out->variants += 1;
+                        if (out->best_ms <= 0.f || best < out->best_ms) {
+                            out->best_ms = best; out->block = block; out->unroll = unroll; out->nontemporal = nt;
+                            out->persistent = persistent; out->interleave = interleave;
+                        }
+                        if (best > out->worst_ms) out->worst_ms = best;
+                    }
+    return SAR_OK;
+}
+
+int sar_probe_streams(sar_ctx* c, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out) {
+    return guarded([&] { return probe_streams_body(c, njobs, jobs, bytes, reps, out); });
+}
+
 int sar_sleep_ticks(sar_ctx* c, float delay_ms, int64_t* ticks) {
     if (!c || !ticks) return set_error(SAR_EINVAL, "null argument");
     if (!(delay_ms >= 0) || !(delay_ms <= kMaxDelayMs)) return set_error(SAR_EINVAL, "delay out of range");
@@ -1161,7 +1239,7 @@ static int plan_body(const sar_schedule* prework, const sar_schedule* main_sched
     HostPlan hp;
     const int rc = hp.make(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units);
     if (rc != SAR_OK) return rc;
-    *out = plan_stats(&hp.c, prework, main_sched, hp.cp, hp.want_column, hp.want_column && hp.want_fused);
+    *out = plan_stats(&hp.c, prework, main_sched, hp.hp.cp, hp.hp.want_column, hp.hp.want_column && hp.hp.want_fused, hp.hp.want_pre);
     return SAR_OK;
 }
 
@@ -1178,11 +1256,11 @@ static int plan_rows_body(const sar_schedule* prework, const sar_schedule* main_
     HostPlan hp;
     const int rc = hp.make(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units);
     if (rc != SAR_OK) return rc;
-    const ColumnPlan& cp = same_launch ? hp.fp : hp.cp;
-    const size_t first = same_launch ? hp.fused_first : hp.col_first;
+    const ColumnPlan& cp = same_launch == 2 ? hp.hp.pp : same_launch ? hp.hp.fp : hp.hp.cp;
+    const size_t first = same_launch == 2 ? hp.hp.pre_first : same_launch ? hp.hp.fused_first : hp.hp.col_first;
     const size_t count = cp.group_begin.empty() ? 0 : cp.group_begin.back();
     if (cp.unsupported || count == 0 || first + count > hp.rows.size())
-        return set_error(SAR_ESTATE, same_launch ? "no plan for pre-work and schedule in one launch" : "no column plan for this schedule and tuning");
+        return set_error(SAR_ESTATE, same_launch == 2 ? "no column plan for the pre-work alone" : same_launch ? "no plan for pre-work and schedule in one launch" : "no column plan for this schedule and tuning");
     auto locate = [&](const char* p, int32_t* rank, uint64_t* off) {
         const uint64_t d = (uint64_t)(p - hp.c.adopted[0]);
         *rank = (int32_t)(d / hp.stride); *off = d % hp.stride;
@@ -1275,8 +1353,11 @@ int run_static_body(int device, void* stream, const sar_schedule* prework, const
     else { (void)hipGetLastError(); c.cu_count = 256; }
 
     std::vector<sar::DevOp> rows; std::vector<char*> ptrs;
-    ColumnPlan cp, fp; uint32_t col_first = 0, fused_first = 0; bool want_column = false, want_fused = false;
-    if ((rc = plan_on_host(&c, prework, main_sched, rows, ptrs, cp, &col_first, &want_column, fp, &fused_first, &want_fused)) != SAR_OK) return rc;
+    HostPlans hp;
+    if ((rc = plan_on_host(&c, prework, main_sched, rows, ptrs, hp)) != SAR_OK) return rc;
+    const ColumnPlan& cp = hp.cp; const ColumnPlan& fp = hp.fp;
+    const uint32_t col_first = hp.col_first, fused_first = hp.fused_first;
+    const bool want_column = hp.want_column, want_fused = hp.want_fused;
 
     // what runs: pre-work and schedule in one launch, or the pre-work's launches followed by the schedule's (one
     // column launch, or one launch per round)

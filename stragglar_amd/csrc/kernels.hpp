@@ -89,6 +89,15 @@ hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t
 // writes 4 * stream_bytes to each of the two windows; stamps[0] / stamps[1] (preset to ~0 / 0) receive the wall-clock
 // ticks of the earliest start and the latest end
 hipError_t launch_region_probe(hipStream_t st, char* a, char* b, uint64_t stream_bytes, unsigned long long* stamps);
+// stream probe (see stream_probe_kernel): up to 8 jobs of up to 8 read and 8 written streams of `bytes` bytes each
+struct ProbeJobs {
+    char* rd[8][8];
+    char* wr[8][8];
+    uint32_t nread[8], nwrite[8];
+    uint32_t njobs, reserved;
+    uint64_t bytes;
+};
+hipError_t launch_stream_probe(hipStream_t st, const ProbeJobs& J, int block, int unroll, bool nontemporal, bool persistent, bool interleave, int compute_units);
 hipError_t launch_sleep(hipStream_t st, uint64_t ticks);
 
 }  // namespace sar

@@ -132,7 +132,7 @@ def test_small_messages_take_the_plan_for_few_items(sarlib):
 def test_prework_and_misaligned_buffers(sarlib):
     S = sarlib.pad_bytes(16 * MIB, 8)
     st = plan(sarlib, "stragglar", 8, S, delay=True)
-    assert st.prework_bytes == 8 * S and st.launches == 2     # one multi-source launch, then the column kernel
+    assert st.prework_bytes == 8 * S and st.launches == 2     # the pre-work as one launch, then the column kernel
     assert st.fused_prework == 1                              # ... or both as one launch when nobody is late
     assert plan(sarlib, "stragglar", 8, S, delay=True, col_fuse_prework=0).fused_prework == 0
     assert plan(sarlib, "stragglar", 8, S, delay=True, executor=0).fused_prework == 0
@@ -143,9 +143,16 @@ def test_prework_and_misaligned_buffers(sarlib):
     # chunk of 4k+2 elements: rows keep their alignment only where the chunk offset happens to allow it
     odd = plan(sarlib, "stragglar", 8, 7 * 4 * 1026, col_latency_plan=0)
     assert 0 <= odd.forwarded_bytes < 42 * 4 * 1026
-    # a schedule with multi-source rows as the main schedule runs one launch per round
+    # a schedule of multi-source rows as the main schedule (the pre-work timed on its own) is one column launch
+    # of 7 work items per column, one launch per round of the multi-source kernel with col_prework = 0 and for
+    # rows that are not whole vectors
     pre = sarlib.builtin("prework_rs", 8)
-    assert sarlib.plan(pre, 8, S).executor == 0
+    st = sarlib.plan(pre, 8, S)
+    assert (st.executor, st.launches, st.col_components, st.col_slots) == (1, 1, 7, 0)
+    assert sarlib.plan(pre, 8, S, col_prework=0).executor == 0
+    assert sarlib.plan(pre, 8, 7 * 4 * 1026).executor == 0
+    rows, ptrs = sarlib.plan_rows(sarlib.builtin("stragglar", 8), 8, S, prework=pre, same_launch=2)
+    assert len(rows) == 7 and all((r.kind, r.nsrc, r.ndst) == (3, 7, 1) for r in rows)
 
 
 def test_plan_argument_checks(sarlib):
