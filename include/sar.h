@@ -49,6 +49,18 @@ enum {
     SAR_OP_MREDUCE = 3      /* dst(s) <- ring-ordered sum over a rank group (the NCCL pre-work collectives)         */
 };
 
+/* why the rank buffers sit where they sit (sar_stats_t.spread_reason) */
+enum {
+    SAR_SPREAD_FOUND = 0,          /* two allocations in different regions of HBM were found: arena_spread = 1 */
+    SAR_SPREAD_OFF = 1,            /* tuning.arena_spread is 0 */
+    SAR_SPREAD_SMALL_PAYLOAD = 2,  /* less than 128 MiB over all ranks: the caches carry the schedule */
+    SAR_SPREAD_UNKNOWN_DEVICE = 3, /* not a 288 GiB MI355X: the regions of this device are not known */
+    SAR_SPREAD_NO_MEMORY = 4,      /* too little free device memory to look for a pair */
+    SAR_SPREAD_NO_PAIR = 5,        /* no candidate was faster against the first allocation than the first against itself */
+    SAR_SPREAD_TOO_LARGE = 6,      /* half the ranks take more than 32 GiB */
+    SAR_SPREAD_ADOPTED = 7         /* caller-owned buffers (sar_adopt_ranks) are taken where they are */
+};
+
 #define SAR_MAX_RANKS 64
 #define SAR_MAX_RANK_BYTES (1ull << 40)   /* largest bytes_per_rank any call accepts */
 
@@ -86,6 +98,11 @@ typedef struct sar_stats_t {
     int32_t arena_spread;          /* 1 if the two halves of the rank buffers lie in different regions of HBM    */
     uint64_t elided_store_bytes;   /* part of algorithmic_bytes that the column executor does not store because a */
                                    /* later row overwrites it and every reader in between takes it from a slot    */
+    int32_t spread_reason;         /* SAR_SPREAD_*: why arena_spread is what it is                                */
+    int32_t spread_candidates;     /* the search for the two allocations (last one this context ran): candidates  */
+    float spread_same_ms;          /* probed, the region probe's time for two windows in one region (the slowest  */
+    float spread_pair_ms;          /* seen) and for the pair that was kept (the slower of its two probes), and    */
+    uint64_t spread_search_bytes;  /* the most device memory held at a time while looking, the pair included      */
 } sar_stats_t;
 
 /* run-time tunables of the executors; sar_get_tuning() reports the defaults */

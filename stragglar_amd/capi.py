@@ -19,6 +19,7 @@ _LIB_PATH = os.path.join(_HERE, "lib", "libsar_hip.so")
 DTYPES = {"f32": 0, "f16": 1, "bf16": 2}
 ELEM_SIZE = {"f32": 4, "f16": 2, "bf16": 2}
 OP_KINDS = {0: "copy", 1: "xreduce", 2: "reduce_into", 3: "mreduce"}
+SPREAD_REASONS = {0: "found", 1: "off", 2: "small payload", 3: "unknown device", 4: "no memory", 5: "no pair", 6: "too large", 7: "adopted"}
 
 
 class SarError(RuntimeError):
@@ -42,7 +43,8 @@ class Stats(ctypes.Structure):
                 ("ops", ctypes.c_int32), ("uses_graph", ctypes.c_int32), ("executor", ctypes.c_int32),
                 ("col_block", ctypes.c_int32), ("col_slots", ctypes.c_int32), ("col_components", ctypes.c_int32),
                 ("forwarded_bytes", ctypes.c_uint64), ("fused_prework", ctypes.c_int32), ("arena_spread", ctypes.c_int32),
-                ("elided_store_bytes", ctypes.c_uint64)]
+                ("elided_store_bytes", ctypes.c_uint64), ("spread_reason", ctypes.c_int32), ("spread_candidates", ctypes.c_int32),
+                ("spread_same_ms", ctypes.c_float), ("spread_pair_ms", ctypes.c_float), ("spread_search_bytes", ctypes.c_uint64)]
 
 
 class PlanRow(ctypes.Structure):

@@ -33,7 +33,8 @@ constexpr uint64_t kArenaAlign = 2ull << 20;   // rank bases on 2 MiB boundaries
 constexpr uint64_t kSpreadMinPayload = 128ull << 20;   // spread arena: from 16 MiB per rank at n = 8 (below, the caches carry the schedule)
 constexpr uint64_t kSpreadHeadroom = 16ull << 30;      // memory left alone while looking for the pair
 constexpr uint64_t kSpreadMinAlloc = 8ull << 30, kSpreadMaxAlloc = 32ull << 30;      // per half; one size serves most payloads
-constexpr uint64_t kSpreadSearch = 112ull << 30;       // candidates held while looking: a region and a bit
+constexpr uint64_t kSpreadSearch = 96ull << 30;        // candidates held while looking, beyond the pair itself: one region
+constexpr float kSpreadFaster = 0.93f;                 // a pair in different regions takes at most this fraction of a pair in one
 constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 streams of this size (beyond what the Infinity Cache absorbs)
 constexpr float kMaxDelayMs = 60000.f;
 
@@ -90,6 +91,10 @@ struct sar_ctx {
     char* pair_hi = nullptr;           // different regions of HBM; kept for the life of the context
     uint64_t pair_bytes = 0;
     bool spread_capable = false;       // the device is one whose regions are known (MI355X, 288 GiB)
+    int spread_reason = SAR_SPREAD_OFF;            // why the ranks sit where they sit (SAR_SPREAD_*)
+    int spread_candidates = 0;                     // what the last search for a pair saw: allocations probed,
+    float spread_same_ms = 0.f, spread_pair_ms = 0.f;      // the probe's time within one region and for the pair kept,
+    uint64_t spread_search_bytes = 0;              // most memory held at a time
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
@@ -172,40 +177,58 @@ float probe_ms(sar_ctx* c, char* a, char* b, int reps) {
 // time in different regions get in each other's way less: the write-heavy schedules here gain 15 to 25 %, and
 // which region a buffer falls in is all that matters, not where in it.  Where an allocation lands physically is
 // the driver's business, so candidates are allocated one after the other and each is timed against the first
-// with a short probe (eight write streams of 128 MiB, four in either allocation: 182-212 us when both lie in
-// the same region, 156-162 us when they do not, on every box seen) until one turns out to lie elsewhere; the
-// others are given back.  Nothing is assumed about the order in which the driver hands out memory, and a wrong
-// verdict costs speed, not correctness: without a pair the caller falls back to one allocation.
-bool find_spread_pair(sar_ctx* c, uint64_t bytes) {
+// with a short probe (eight write streams of 128 MiB, four in either allocation) until one turns out to lie
+// elsewhere; the others are given back.  The yardstick is the probe's own time for two windows that do share a
+// region -- two neighbouring windows of the first allocation --, not a fixed figure: elsewhere means at most
+// kSpreadFaster of that, twice, on different windows of both (measured: 154-162 us against 175-212 us for
+// candidates in the first allocation's region, 181 us for its own two windows).  At most one region's worth of
+// candidates is held at a time beyond the pair.  Nothing is assumed about the order in which the driver hands
+// out memory, and a wrong verdict costs speed, not correctness: without a pair the caller falls back to one
+// allocation.  Returns a SAR_SPREAD_* reason.
+int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     const uint64_t window = 4 * kProbeStream;
-    const float elsewhere_ms = (float)(8.0 * (double)kProbeStream / 6.3e9);      // the probe's 1 GiB at 6.3 TB/s: 170 us
-    if (bytes < 2 * window) return false;
+    c->spread_candidates = 0; c->spread_same_ms = c->spread_pair_ms = 0.f; c->spread_search_bytes = 0;
+    if (bytes < 2 * window) return SAR_SPREAD_NO_PAIR;
     size_t free_b = 0, total_b = 0;
-    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); return false; }
-    if (free_b < 4 * bytes + kSpreadHeadroom) return false;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); return SAR_SPREAD_NO_MEMORY; }
+    if (free_b < 4 * bytes + kSpreadHeadroom) return SAR_SPREAD_NO_MEMORY;
     // enough candidates to cross a region boundary from anywhere, no more
     const uint64_t budget = std::min<uint64_t>((uint64_t)free_b - kSpreadHeadroom, kSpreadSearch + 2 * bytes);
     std::vector<char*> held;
-    try { held.reserve((size_t)(budget / bytes) + 1); } catch (const std::bad_alloc&) { return false; }      // no allocation below
+    try { held.reserve((size_t)(budget / bytes) + 1); } catch (const std::bad_alloc&) { return SAR_SPREAD_NO_MEMORY; }      // no allocation below
+    // The first allocation, and the yardstick: the probe's time for two neighbouring windows at its start, which
+    // share a region.  Should a boundary run through the allocation (its two ends then probe like a pair in
+    // different regions), it stays held as a spacer and the one behind it takes its place.
     char* lo = nullptr;
-    if (hipMalloc((void**)&lo, bytes) != hipSuccess) { (void)hipGetLastError(); return false; }
+    float same = -1.f;
+    uint64_t used = 0;
+    for (int attempt = 0; attempt < 2 && used + bytes <= budget; ++attempt) {
+        if (hipMalloc((void**)&lo, bytes) != hipSuccess) { (void)hipGetLastError(); lo = nullptr; break; }
+        used += bytes;
+        same = probe_ms(c, lo, lo + window, 3);
+        const float ends = probe_ms(c, lo, lo + bytes - window, 3);
+        if (same > 0.f && ends > 0.f && ends < kSpreadFaster * same && attempt == 0) { held.push_back(lo); lo = nullptr; continue; }
+        break;
+    }
     char* hi = nullptr;
-    for (uint64_t used = bytes; used + bytes <= budget; used += bytes) {
+    for (; lo && same > 0.f && used + bytes <= budget; used += bytes) {
         char* cand = nullptr;
         if (hipMalloc((void**)&cand, bytes) != hipSuccess) { (void)hipGetLastError(); break; }
+        c->spread_candidates += 1;
         const float t = probe_ms(c, lo, cand, 3);
         if (t < 0.f) { (void)hipFree(cand); break; }
-        // elsewhere if fast twice, on different windows of both
-        if (t < elsewhere_ms) {
+        if (t < kSpreadFaster * same) {
             const float t2 = probe_ms(c, lo + bytes - window, cand + bytes - window, 3);
-            if (t2 > 0.f && t2 < elsewhere_ms) { hi = cand; break; }
+            if (t2 > 0.f && t2 < kSpreadFaster * same) { hi = cand; c->spread_pair_ms = std::max(t, t2); used += bytes; break; }
         }
         held.push_back(cand);
     }
+    c->spread_same_ms = std::max(same, 0.f);
+    c->spread_search_bytes = used;
     for (char* p : held) (void)hipFree(p);
-    if (!hi) { (void)hipFree(lo); return false; }
+    if (!hi) { if (lo) (void)hipFree(lo); return lo ? SAR_SPREAD_NO_PAIR : SAR_SPREAD_NO_MEMORY; }
     c->pair_lo = lo; c->pair_hi = hi; c->pair_bytes = bytes;
-    return true;
+    return SAR_SPREAD_FOUND;
 }
 
 void drop_ranks(sar_ctx* c) {
@@ -598,6 +621,8 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     st.elided_store_bytes = column ? cp.elided_bytes : 0;
     st.fused_prework = fused ? 1 : 0;
     st.arena_spread = c->spread() ? 1 : 0;
+    st.spread_reason = c->spread_reason; st.spread_candidates = c->spread_candidates;
+    st.spread_same_ms = c->spread_same_ms; st.spread_pair_ms = c->spread_pair_ms; st.spread_search_bytes = c->spread_search_bytes;
     return st;
 }
 
@@ -795,12 +820,15 @@ static int alloc_ranks_body(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtyp
     // the room to look for such a pair; otherwise the ranks sit back to back.
     const int half = (n + 1) / 2;
     const uint64_t payload = stride * (uint64_t)n;
-    bool spread = c->tune.arena_spread != 0 && c->spread_capable && payload >= kSpreadMinPayload;
-    if (spread) {
+    int reason = !c->tune.arena_spread ? SAR_SPREAD_OFF : !c->spread_capable ? SAR_SPREAD_UNKNOWN_DEVICE :
+                 payload < kSpreadMinPayload ? SAR_SPREAD_SMALL_PAYLOAD : SAR_SPREAD_FOUND;
+    if (reason == SAR_SPREAD_FOUND) {
         uint64_t need = kSpreadMinAlloc;
         while (need < stride * (uint64_t)half) need <<= 1;
-        if (c->pair_bytes < need) { drop_pair(c); spread = need <= kSpreadMaxAlloc && find_spread_pair(c, need); }
+        if (c->pair_bytes < need) { drop_pair(c); reason = need <= kSpreadMaxAlloc ? find_spread_pair(c, need) : SAR_SPREAD_TOO_LARGE; }
     }
+    const bool spread = reason == SAR_SPREAD_FOUND;
+    c->spread_reason = reason;
     if (spread) {
         c->arena = c->pair_lo; c->arena_hi = c->pair_hi; c->split = half;
     } else {
@@ -861,6 +889,7 @@ static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_
     drop_ranks(c);
     for (int r = 0; r < n; ++r) c->adopted.push_back((char*)device_ptrs[r]);
     c->n = n; c->dtype = dtype; c->bytes_per_rank = bytes_per_rank; c->stride = 0;
+    c->spread_reason = SAR_SPREAD_ADOPTED;
     return SAR_OK;
 }
 

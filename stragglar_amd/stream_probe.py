@@ -1,0 +1,83 @@
+#!/usr/bin/env python3
+"""What the memory system delivers for the stream mixes of an emulated AllReduce: the yardstick for the data kernels.
+
+    python -m stragglar_amd.stream_probe [--ranks 8] [--mib 256] [--dtype f32] [--reps 5] [--spread 1]
+
+The rank buffers are allocated as for a run (padded as pad_buffers.py pads, placed by sar_alloc_ranks) and the
+library's stream probe -- a kernel that only loads, adds and stores, tried in 36 or 72 launch shapes, the fastest
+counted -- moves the same bytes between the same addresses as
+
+    exchanges   the reduce steps of the StragglAR table alone: per chunk r, rank r's and the straggler's chunk r
+                are read and their sum is written over both (2 reads + 2 writes in place; what exchange +
+                reduce_add of allreduce_8GPU.cu:564-578 comes to on one GPU)
+    one         one such exchange on its own (the first round of the table)
+    schedule    the whole table once re-reads are served on chip: the two cold reads of every chunk and the sum
+                written to every rank (2 reads + n writes)
+    prework     the in-place ReduceScatter of the n-1 ranks that are on time (n-1 reads + 1 write per chunk)
+    copy/read/write   one buffer copied to another; all buffers read; all buffers written
+
+One line per mix: microseconds, GB/s, fraction of the 8 TB/s peak, the fastest shape and the slowest shape's time.
+"""
+import argparse
+import sys
+
+from . import capi
+
+PEAK = 8000.0
+
+
+def mixes(n, chunk, whole):
+    s = n - 1
+    out = [("exchanges", [([r, s], [r, s], r * chunk) for r in range(s)], chunk),
+           ("one", [([0, s], [0, s], 0)], chunk),
+           ("schedule", [([r, s], list(range(n)), r * chunk) for r in range(s)], chunk),
+           ("prework", [([(r + q) % s for q in range(1, s + 1)], [r], r * chunk) for r in range(s)], chunk),
+           ("copy", [([0], [n // 2], 0)], whole),
+           ("read", [(list(range(n)), [], 0)], whole),
+           ("write", [([], list(range(n)), 0)], whole)]
+    return [m for m in out if len(m[1]) <= 8 and all(len(rd) <= 8 and len(wr) <= 8 for rd, wr, _ in m[1])]
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--ranks", type=int, default=8)
+    ap.add_argument("--mib", type=float, default=256.0, help="unpadded MiB per rank")
+    ap.add_argument("--dtype", default="f32", choices=sorted(capi.DTYPES))
+    ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--spread", type=int, default=1, choices=[0, 1], help="0 = all rank buffers back to back in one allocation")
+    ap.add_argument("--mix", default="", help="comma-separated subset of the mixes")
+    args = ap.parse_args(argv)
+    lib = capi.load_library()
+    n = args.ranks
+    if n < 3 or n > 9:
+        print("3 to 9 ranks, please: a probe job holds at most 8 streams a side", file=sys.stderr)
+        return 2
+    es = capi.ELEM_SIZE[args.dtype]
+    nbytes = lib.pad_bytes(int(args.mib * (1 << 20)), n)
+    chunk = (nbytes // es // (n - 1)) * es
+    chunk -= chunk % 16
+    ctx = lib.context(0)
+    ctx.set_tuning(arena_spread=args.spread)
+    ctx.alloc_ranks(n, nbytes, args.dtype)
+    for r in range(n):
+        ctx.fill_uniform(r, 1 + r, -1.0, 1.0)
+    ctx.prepare(lib.builtin("ring", n))                     # only to read the placement from the stats
+    st = ctx.stats()
+    print("n=%d, %d B per rank (%s), chunk %d B, rank buffers in two regions of HBM: %d (%s)"
+          % (n, nbytes, args.dtype, chunk, st.arena_spread, capi.SPREAD_REASONS.get(st.spread_reason, "?")))
+    print("mix,streams,bytes_moved,us,GB/s,frac_of_8TBps,best_shape(block/vectors/streaming/resident/turns),slowest_shape_us,shapes")
+    want = [m for m in args.mix.split(",") if m]
+    for name, jobs, size in mixes(n, chunk, nbytes - nbytes % 16):
+        if want and name not in want:
+            continue
+        res = ctx.probe_streams(jobs, size, args.reps)
+        rd, wr, _ = jobs[0]
+        print("%s,%d x (%dR+%dW),%d,%.1f,%.0f,%.3f,%d/%d/%d/%d/%d,%.1f,%d"
+              % (name, len(jobs), len(rd), len(wr), res.bytes_moved, res.best_ms * 1e3, res.gbps, res.gbps / PEAK,
+                 res.block, res.unroll, res.nontemporal, res.persistent, res.interleave, res.worst_ms * 1e3, res.variants), flush=True)
+    ctx.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -12,7 +12,8 @@ size -> unflatten).
 Here all ranks are emulated in ONE process on ONE GPU: the caller hands over
 one tensor per emulated rank and the library works on those tensors in place
 (``sar_adopt_ranks``: no copy into an arena).  torch is used for the tensors
-only; the schedule runs in the HIP library.
+only; the schedule runs in the HIP library.  ``stragglar_amd.c10d_backend``
+puts the same group behind ``torch.distributed.all_reduce``.
 """
 from __future__ import annotations
 
@@ -23,6 +24,22 @@ from . import capi
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _TORCH_DTYPES = {"torch.float32": "f32", "torch.float16": "f16", "torch.bfloat16": "bf16"}
+
+
+def padded_numel(numel: int, world_size: int, elem_size: int, parts: Optional[int] = None) -> int:
+    """Element count of a flat buffer padded the way the reference's callers pad theirs (example.py:19:
+    ``ceil(bytes / (1024 * 7)) * 1024 * 7`` for 8 ranks): chunks of whole KiB, so every chunk starts on a
+    16-byte boundary.  ``parts`` = chunks per buffer (world_size - 1 for StragglAR, the default)."""
+    parts = world_size - 1 if parts is None else parts
+    unit = 1024 * parts
+    return -(-(numel * elem_size) // unit) * unit // elem_size
+
+
+class _DeviceArray:
+    """Device memory owned by the library, described for ``torch.as_tensor`` (no copy)."""
+
+    def __init__(self, ptr: int, numel: int, typestr: str):
+        self.__cuda_array_interface__ = {"shape": (numel,), "typestr": typestr, "data": (ptr, False), "version": 2}
 
 
 class EmulatedGroup:
@@ -66,17 +83,45 @@ class EmulatedGroup:
     def close(self):
         self._ctx.close()
 
+    def rank_tensors(self, numel: int, dtype) -> List:
+        """One flat tensor of ``numel`` elements per emulated rank, in memory the library allocates and places
+        itself (``sar_alloc_ranks``: from 128 MiB over all ranks, half the ranks in another region of HBM than the
+        rest, which is worth 15 to 25 % of the bandwidth and which tensors that torch allocated next to each other
+        cannot have).  The tensors alias the group's memory: they are valid until the next ``rank_tensors`` call or
+        ``close``.  ``all_reduce`` on them skips the adoption step."""
+        import torch
+        name = _TORCH_DTYPES.get(str(dtype))
+        if name is None:
+            raise TypeError("unsupported dtype %s" % dtype)
+        es = capi.ELEM_SIZE[name]
+        self._ctx.alloc_ranks(self.n, numel * es, name)
+        order = list(range(self.n))
+        order[self.straggler], order[self.n - 1] = order[self.n - 1], order[self.straggler]
+        typestr = {"f32": "<f4", "f16": "<f2", "bf16": "<i2"}[name]
+        out = [None] * self.n
+        ptrs = []
+        for k, i in enumerate(order):                   # schedule rank k is the caller's rank order[k]
+            ptr = self._ctx.rank_pointer(k)
+            ptrs.append(ptr)
+            t = torch.as_tensor(_DeviceArray(ptr, numel, typestr), device="cuda:%d" % self.device)
+            out[i] = t.view(torch.bfloat16) if name == "bf16" else t
+        self._ctx.prepare(self._main, self._prework)
+        self._key = (tuple(ptrs), numel * es, name)
+        return out
+
     def _order(self, tensors):
         """Rank order seen by the schedule: the straggler takes the last place."""
         order = list(range(self.n))
         order[self.straggler], order[self.n - 1] = order[self.n - 1], order[self.straggler]
         return [tensors[i] for i in order]
 
-    def all_reduce(self, tensors: Sequence, delay_ms: float = 0.0) -> float:
+    def all_reduce(self, tensors: Sequence, delay_ms: float = 0.0, strict: bool = True) -> float:
         """Sum-AllReduce in place: ``tensors[r]`` is rank r's flat buffer.  Afterwards every tensor holds the
         sum.  The element count must divide by world_size-1 for StragglAR (world_size for ring / rhd), as in the
-        reference, whose callers pad their buffers (example.py:19).  ``delay_ms > 0`` makes the straggler late
-        by that much.  Returns the elapsed milliseconds."""
+        reference, whose callers pad their buffers (example.py:19); with ``strict=False`` a count that does not
+        divide is taken as the reference takes it: chunk = numel // parts, and the elements behind the last chunk
+        are left as they are (allreduce_stragglar, dummy.cpp:265).  ``delay_ms > 0`` makes the straggler late by
+        that much.  Returns the elapsed milliseconds."""
         import torch
         if len(tensors) != self.n:
             raise ValueError("need one tensor per emulated rank")
@@ -88,7 +133,7 @@ class EmulatedGroup:
             if not t.is_cuda or t.device.index != self.device or not t.is_contiguous() or t.dtype != t0.dtype or t.numel() != t0.numel():
                 raise ValueError("rank tensors must be contiguous CUDA tensors of one dtype and size on device %d" % self.device)
         parts = self._main.parts
-        if t0.numel() % parts:
+        if strict and t0.numel() % parts:
             raise ValueError("element count %d does not divide into %d chunks: pad the buffer" % (t0.numel(), parts))
         ordered = self._order(tensors)
         nbytes = t0.numel() * t0.element_size()
@@ -110,7 +155,9 @@ class EmulatedGroup:
         flats = []
         for grads in per_rank_grads:
             flat = torch.cat([g.reshape(-1) for g in grads])
-            pad = (-flat.numel()) % parts
+            # padded as example.py:19 pads: chunks of whole KiB, so that every chunk is a whole number of 16-byte
+            # vectors on a vector boundary (the rows then run as vectors, pre-work and schedule as one launch)
+            pad = padded_numel(flat.numel(), self.n, flat.element_size(), parts) - flat.numel()
             if pad:
                 flat = torch.cat([flat, flat.new_zeros(pad)])
             flats.append(flat.contiguous())

@@ -95,6 +95,67 @@ def test_reducescatter_twin():
         assert m and int(m.group(1)) == i + 1
 
 
+def test_reducescatter_result_through_the_c_abi(sarlib, gpu_ctx, oracle):
+    """What the twin times, on the same size: rank i filled with i+1 as reducescatter.cu:97-101 fills it, then the
+    in-place ReduceScatter of ranks 0-6 -- chunk r of rank r becomes 1 + ... + 7 = 28, everything else stays --
+    and on seeded inputs the checker's bits, with the multi-source kernel and with the column kernel."""
+    import numpy as np
+    from conftest import assert_bits_equal, make_inputs
+    n, nbytes = 8, 1053696
+    elems, chunk = nbytes // 4, nbytes // 4 // 7
+    rs = sarlib.builtin("prework_rs", n)
+    for col_prework in (1, 0):
+        gpu_ctx.set_tuning(**dict(gpu_ctx.default_tuning, col_prework=col_prework))
+        gpu_ctx.alloc_ranks(n, nbytes, "f32")
+        gpu_ctx.prepare(rs)
+        assert gpu_ctx.stats().executor == col_prework
+        for r in range(n):
+            gpu_ctx.fill_const(r, r + 1.0)
+        gpu_ctx.run(-1.0)
+        for r in range(n):
+            want = np.full(elems, r + 1.0, np.float32)
+            if r < n - 1:
+                want[r * chunk:(r + 1) * chunk] = 28.0
+            assert np.array_equal(gpu_ctx.download(r), want), "rank %d" % r
+        inputs = make_inputs(n, elems, "f32", seed=21)
+        for r, x in enumerate(inputs):
+            gpu_ctx.upload(r, x)
+        gpu_ctx.run(-1.0)
+        want = [x.copy() for x in inputs]
+        oracle.prework_reduce_scatter(want, "f32")
+        for r in range(n):
+            assert_bits_equal(gpu_ctx.download(r), want[r], "col_prework %d rank %d" % (col_prework, r))
+    gpu_ctx.set_tuning(**gpu_ctx.default_tuning)
+
+
+def test_delay_sweep_tool():
+    """python -m stragglar_amd.delay_sweep: the reference's delay mode for the four algorithms
+    (allreduce_8GPU.cu:115-137,201-219,535-553,876-898).  A delay that covers the pre-work takes it off the
+    critical path for stragglar and direct -- after the straggler has arrived they finish sooner than without a
+    delay -- while ring and rhd, which have no pre-work, take as long as ever."""
+    import sys
+    p = run(sys.executable, "-m", "stragglar_amd.delay_sweep", "--mib", "64", "--delays", "0,3", "--iters", "5")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = p.stdout.splitlines()
+    assert lines[0] == "algorithm,buffer_size_bytes,delay,runtime_ms,runtime_minus_delay_ms,BW(GB/s)"
+    rows = {}
+    for l in lines[1:]:
+        if l.startswith("#"):
+            continue
+        alg, nbytes, delay, ms, rest, bw = l.split(",")
+        delay, ms, rest, bw = float(delay), float(ms), float(rest), float(bw)
+        assert ms >= delay and abs(rest - (ms - delay)) < 2e-3 and rest > 0
+        assert abs(bw - int(nbytes) / 2 ** 30 * 1000 / rest) <= bw * (0.0011 / rest + 1e-3) + 0.002
+        rows[(alg, delay)] = rest
+    assert sorted(rows) == sorted((a, d) for a in ("stragglar", "ring", "rhd", "direct") for d in (0.0, 3.0))
+    for alg in ("stragglar", "direct"):
+        assert rows[(alg, 3.0)] < rows[(alg, 0.0)], (alg, rows)
+    for alg in ("ring", "rhd"):
+        assert rows[(alg, 3.0)] > 0.85 * rows[(alg, 0.0)], (alg, rows)
+    assert rows[("stragglar", 3.0)] < rows[("ring", 3.0)]
+    assert any(l.startswith("# delay 3.000 ms:") for l in lines)
+
+
 @pytest.mark.parametrize("extra", [[], ["--executor", "0"], ["--forward", "0"], ["--alg", "ring", "--no-cpu"]])
 def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     """bench.py end to end (at 16 MiB per rank so that it takes a second): exactly one JSON line on stdout, the
@@ -115,6 +176,19 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s" and "traffic" in roof
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert rec["ranks_identical_after_run"] is True
+    # value is the HBM rate (bytes that reach memory), the rows' own bytes are reported beside it
+    assert abs(rec["value"] - rec["memory_bytes_per_step"] / rec["ms_per_step"] / 1e6) <= 0.002 * rec["value"]
+    assert abs(rec["algorithmic_GBps"] - rec["algorithmic_bytes_per_step"] / rec["ms_per_step"] / 1e6) <= 0.002 * rec["algorithmic_GBps"]
+    assert rec["memory_bytes_per_step"] == rec["algorithmic_bytes_per_step"] - rec["forwarded_bytes_per_step"] - rec["elided_store_bytes_per_step"]
+    assert abs(roof["achieved"] - roof["memory_bytes_per_launch"] / roof["mean_launch_ms"] / 1e6) <= 0.002 * roof["achieved"]
+    assert rec["host"]["logical_cpus"] >= 1
+    if "--alg" not in extra:
+        assert sorted(rec["comparators"]) == ["direct", "rhd", "ring"]
+        for leg in rec["comparators"].values():
+            assert leg["ranks_identical_after_run"] is True and leg["ms_per_step"] > 0 and leg["memory_side_GBps"] > 0
+            assert leg["bit_exact_vs_cpu_checker"] is True
+    if "--alg" not in extra and "--forward" not in extra and "--executor" not in extra:
+        assert 0 < rec["stream_ceiling"]["GBps"] and rec["stream_ceiling"]["shapes_tried"] == 72
     if "--no-cpu" not in extra:
         base = rec["cpu_baseline"]
         assert base["kind"] == "port" and base["cores"] == 1 and base["value"] > 0 and base["unit"] == "GB/s" and base["sample"]

@@ -759,7 +759,19 @@ def test_spread_arena(gpu_ctx, sarlib, oracle):
         gpu_ctx.restore()
         assert gpu_ctx.ranks_identical((elems // 7) * 7)
         assert_bits_equal(gpu_ctx.download(5), want[5], "after restore")
-    assert seen[2:4] == [0, 0] and seen[0] == seen[1] == seen[4] == seen[5]      # 1 where the device has the room
+    assert seen[2:4] == [0, 0] and seen[0] == seen[1] == seen[4] == seen[5]
+    # On the device this build is for (288 GiB) the two allocations must have been found: a probe that stopped
+    # telling the regions apart would pass every parity test and cost a fifth of the bandwidth unnoticed.
+    from stragglar_amd.capi import SPREAD_REASONS
+    st = gpu_ctx.stats()
+    why = "arena_spread %d, reason '%s', %d candidates probed, probe %.1f us within a region, %.1f us for the pair, %.1f GiB held while looking" % (
+        st.arena_spread, SPREAD_REASONS.get(st.spread_reason, "?"), st.spread_candidates, st.spread_same_ms * 1e3, st.spread_pair_ms * 1e3,
+        st.spread_search_bytes / 2.0 ** 30)
+    print(why)
+    if st.spread_reason != 3:                    # 3: not a 288 GiB device, regions unknown
+        assert seen[0] == 1 and st.spread_reason == 0, why
+        assert 0 < st.spread_pair_ms < 0.93 * st.spread_same_ms, why
+        assert st.spread_search_bytes <= (96 + 2 * 8 + 1) << 30, why
     # small payloads stay back to back
     small = make_inputs(n, 7 * 8 * 100, dtype, seed=78)
     gpu_ctx.set_tuning(arena_spread=1)

@@ -147,3 +147,80 @@ def test_rank_tensors_that_start_off_the_vector_boundary(oracle, dtype, name, sh
                 assert torch.all(pool[lo:lo + shift] == 0) and torch.all(pool[lo + shift + numel:hi] == 0)
         finally:
             group.close()
+
+
+@pytest.fixture()
+def c10d_group():
+    import torch.distributed as dist
+    import stragglar_amd.c10d_backend as sb
+    sb.configure(straggler_rank=6)                       # STRAGGLER_RANK of the reference (dummy.cpp:157, dp.py:22)
+    dist.init_process_group(sb.BACKEND_NAME, store=dist.HashStore(), rank=0, world_size=1)
+    yield sb
+    dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.float32, "f32"), (torch.float16, "f16"), (torch.bfloat16, "bf16")])
+def test_dist_all_reduce_reaches_the_emulation(c10d_group, oracle, dtype, name):
+    """torch.distributed.all_reduce on a backend registered by name, as the reference's callers use theirs
+    (example.py:16-30): the rows of one [8, numel] tensor are the emulated ranks, the straggler is rank 6 and
+    takes the last place, and every row ends with the checker's bits."""
+    import torch.distributed as dist
+    n = 8
+    numel = c10d_group.padded_numel(100000, n, dtype.itemsize)          # example.py:19
+    assert (numel * dtype.itemsize) % (1024 * 7) == 0
+    g = torch.Generator(device="cpu").manual_seed(5)
+    y = (torch.rand(n, numel, generator=g, dtype=torch.float32) * 2 - 1).to(dtype).cuda()
+    inputs = [to_np_bits(y[r]).copy() for r in range(n)]
+    work = dist.all_reduce(y, async_op=True)
+    assert work.is_completed() and work.wait()
+    order = list(range(n))
+    order[6], order[7] = order[7], order[6]
+    want = [inputs[i].copy() for i in order]
+    oracle.run("stragglar", want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+    for k, i in enumerate(order):
+        assert_bits_equal(to_np_bits(y[i]), want[k], "rank %d" % i)
+    # a second call on the same tensor sums the sums (dist.all_reduce without async_op returns nothing)
+    assert dist.all_reduce(y) is None
+    oracle.run("stragglar", want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+    for k, i in enumerate(order):
+        assert_bits_equal(to_np_bits(y[i]), want[k], "second call, rank %d" % i)
+
+
+def test_dist_all_reduce_leaves_the_tail_as_the_reference_does(c10d_group, oracle):
+    """chunkSize = numel / (size - 1) in allreduce_stragglar (dummy.cpp:265): what lies behind the last chunk is
+    not reduced.  Other rank counts get groups of their own."""
+    import torch.distributed as dist
+    for n, numel in ((8, 7 * 300 + 5), (4, 3 * 1000 + 2)):
+        y = torch.arange(n * numel, dtype=torch.float32).reshape(n, numel).cuda() % 17
+        before = y.clone()
+        dist.all_reduce(y)
+        body = (numel // (n - 1)) * (n - 1)
+        assert torch.equal(y[:, body:], before[:, body:])
+        assert torch.equal(y[:, :body], before[:, :body].sum(dim=0, keepdim=True).expand(n, body))     # small integers: exact in any order
+
+
+def test_rank_tensors_are_placed_by_the_library(oracle):
+    """EmulatedGroup.rank_tensors: torch tensors over memory that sar_alloc_ranks allocated and placed (half the
+    ranks in another region of HBM from 128 MiB over all ranks), worked on without adoption."""
+    from stragglar_amd.torch_emulation import EmulatedGroup
+    n, numel = 8, 7 * 8 * 160000                     # 9 M elements per rank: 143 MB over all ranks in bf16, 287 MB in fp32
+    group = EmulatedGroup(n, straggler_rank=6)
+    try:
+        for dtype, name in ((torch.float32, "f32"), (torch.bfloat16, "bf16")):
+            tensors = group.rank_tensors(numel, dtype)
+            assert len(tensors) == n and all(t.dtype == dtype and t.numel() == numel and t.is_cuda for t in tensors)
+            g = torch.Generator(device="cpu").manual_seed(9)
+            for t in tensors:
+                t.copy_((torch.rand(numel, generator=g, dtype=torch.float32) * 2 - 1).to(dtype))
+            inputs = [to_np_bits(t).copy() for t in tensors]
+            group.all_reduce(tensors)
+            st = group._ctx.stats()
+            assert st.spread_reason in (0, 3) and st.arena_spread == (1 if st.spread_reason == 0 else 0)      # 3: not a 288 GiB device
+            order = list(range(n))
+            order[6], order[7] = order[7], order[6]
+            want = [inputs[i].copy() for i in order]
+            oracle.run("stragglar", want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+            for k, i in enumerate(order):
+                assert_bits_equal(to_np_bits(tensors[i]), want[k], "%s rank %d" % (name, i))
+    finally:
+        group.close()
