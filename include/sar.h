@@ -153,7 +153,8 @@ typedef struct sar_tuning_t {
     int32_t col_fuse_chains; /* column executor: 1 = a chain of one-sided reduces whose partial sums are  */
                           /*     neither stored nor read by anyone else (a ring's reduce-scatter)   */
                           /*     runs as one multi-source row, all its cold operands loaded together */
-                          /*     (in the plan for few work items, where the round trips are the cost) */
+                          /*     (in the plan for few work items, where the round trips are the cost;  */
+                          /*     2 = in every plan: measured 1 to 7 % slower where memory is the bound)      */
     int32_t col_fuse_copies; /* column executor: 1 = copies of a value that an earlier row of the work   */
                           /*     item still holds are issued by that row as extra stores, and the    */
                           /*     copy rows (with their round boundaries) go away, where that was     */

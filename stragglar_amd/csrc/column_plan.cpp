@@ -51,7 +51,7 @@ public:
         if (fwd.nslots && env_.tune.col_elide_stores) {
             mark_dead_stores(fwd);
             // (in the bandwidth regime the chain is bound by memory either way: measured equal to 2 % slower)
-            if (env_.tune.col_fuse_chains && plan_.staged) fuse_chains(fwd);
+            if (env_.tune.col_fuse_chains == 2 || (env_.tune.col_fuse_chains == 1 && plan_.staged)) fuse_chains(fwd);
         }
         const bool pays = !plan_.staged || env_.tune.col_slots != 0 || !fwd.nslots || slots_pay_when_staged(fwd);
         const uint32_t rows_before = (uint32_t)before.cr.size();

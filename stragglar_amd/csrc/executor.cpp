@@ -635,7 +635,7 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_forward == 0 || t.col_forward == 1) && t.col_slots >= 0 && t.col_slots <= 255 &&
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
-           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && (t.col_fuse_chains == 0 || t.col_fuse_chains == 1) && t.col_fuse_copies >= 0 && t.col_fuse_copies <= 2 &&
+           (t.col_elide_stores == 0 || t.col_elide_stores == 1) && t.col_fuse_chains >= 0 && t.col_fuse_chains <= 2 && t.col_fuse_copies >= 0 && t.col_fuse_copies <= 2 &&
            (t.arena_spread == 0 || t.arena_spread == 1) && (t.col_prework == 0 || t.col_prework == 1);
 }
 

@@ -14,6 +14,9 @@ counted -- moves the same bytes between the same addresses as
     schedule    the whole table once re-reads are served on chip: the two cold reads of every chunk and the sum
                 written to every rank (2 reads + n writes)
     prework     the in-place ReduceScatter of the n-1 ranks that are on time (n-1 reads + 1 write per chunk)
+    ring        what ring and halving-doubling send to memory once partial sums stay on chip: per chunk of S/n every
+                rank's copy is read once and written once (n reads + n writes in place)
+    direct      the same for direct: rank 0's and the straggler's whole buffers are read, the sum goes to every rank
     copy/read/write   one buffer copied to another; all buffers read; all buffers written
 
 One line per mix: microseconds, GB/s, fraction of the 8 TB/s peak, the fastest shape and the slowest shape's time.
@@ -26,12 +29,16 @@ from . import capi
 PEAK = 8000.0
 
 
-def mixes(n, chunk, whole):
+def mixes(n, chunk, whole, es):
     s = n - 1
+    nth = (whole // es // n) * es
+    nth -= nth % 16
     out = [("exchanges", [([r, s], [r, s], r * chunk) for r in range(s)], chunk),
            ("one", [([0, s], [0, s], 0)], chunk),
            ("schedule", [([r, s], list(range(n)), r * chunk) for r in range(s)], chunk),
            ("prework", [([(r + q) % s for q in range(1, s + 1)], [r], r * chunk) for r in range(s)], chunk),
+           ("ring", [(list(range(n)), list(range(n)), c * nth) for c in range(n)], nth),
+           ("direct", [([0, s], list(range(n)), 0)], whole),
            ("copy", [([0], [n // 2], 0)], whole),
            ("read", [(list(range(n)), [], 0)], whole),
            ("write", [([], list(range(n)), 0)], whole)]
@@ -49,8 +56,8 @@ def main(argv=None) -> int:
     args = ap.parse_args(argv)
     lib = capi.load_library()
     n = args.ranks
-    if n < 3 or n > 9:
-        print("3 to 9 ranks, please: a probe job holds at most 8 streams a side", file=sys.stderr)
+    if n < 3 or n > 8:
+        print("3 to 8 ranks, please: a probe job holds at most 8 streams a side", file=sys.stderr)
         return 2
     es = capi.ELEM_SIZE[args.dtype]
     nbytes = lib.pad_bytes(int(args.mib * (1 << 20)), n)
@@ -67,7 +74,7 @@ def main(argv=None) -> int:
           % (n, nbytes, args.dtype, chunk, st.arena_spread, capi.SPREAD_REASONS.get(st.spread_reason, "?")))
     print("mix,streams,bytes_moved,us,GB/s,frac_of_8TBps,best_shape(block/vectors/streaming/resident/turns),slowest_shape_us,shapes")
     want = [m for m in args.mix.split(",") if m]
-    for name, jobs, size in mixes(n, chunk, nbytes - nbytes % 16):
+    for name, jobs, size in mixes(n, chunk, nbytes - nbytes % 16, es):
         if want and name not in want:
             continue
         res = ctx.probe_streams(jobs, size, args.reps)
