@@ -861,7 +861,7 @@ __global__ __launch_bounds__(1024) void stream_probe_kernel(ProbeJobs J, uint32_
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint64_t i = first + (uint64_t)u * blockDim.x;
-            v[u] = f4{1.f, 2.f, 3.f, 4.f};
+            v[u] = R ? f4{0.f, 0.f, 0.f, 0.f} : f4{1.f, 2.f, 3.f, 4.f};
             if (whole || i < nvec) {
 #pragma unroll
                 for (int k = 0; k < R; ++k) v[u] += ld16<NT>(J.rd[job][k] + (i << 4));

@@ -156,6 +156,38 @@ def test_delay_sweep_tool():
     assert any(l.startswith("# delay 3.000 ms:") for l in lines)
 
 
+def test_measurement_tools_run():
+    """python -m stragglar_amd.stream_probe / hbm_regions at small sizes: one CSV line per mix, a square map."""
+    import sys
+    p = run(sys.executable, "-m", "stragglar_amd.stream_probe", "--mib", "4", "--reps", "1")
+    assert p.returncode == 0, p.stdout + p.stderr
+    rows = [l.split(",") for l in p.stdout.splitlines()[2:]]
+    assert [r[0] for r in rows] == ["exchanges", "one", "schedule", "prework", "ring", "direct", "copy", "read", "write"]
+    assert all(len(r) == 9 and float(r[3]) > 0 and float(r[4]) > 0 for r in rows)
+    assert rows[2][1] == "7 x (2R+8W)" and int(rows[2][2]) * 4 == int(rows[0][2]) * 10         # 10 streams a job against 4
+    p = run(sys.executable, "-m", "stragglar_amd.hbm_regions", "--gib", "16", "--slot-gib", "1", "--stream-mib", "8", "--reps", "1")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = p.stdout.splitlines()
+    grid = [l.split() for l in lines[3:7]]
+    assert all(len(g) == 5 for g in grid) and [g[0] for g in grid] == ["0", "4", "8", "12"]
+    assert grid[0][2] == grid[1][1]                                  # the map is symmetric: a pair is measured once
+    assert any(l.startswith("region of every group:") for l in lines)
+
+
+def test_cli_runs_a_row_list_that_is_no_allreduce():
+    """--schedule with a row list, --nocheck, --executor: the exchanges of the n=8 table alone, both executors."""
+    rows = os.path.join(ROOT, "stragglar_amd", "schedules", "exchanges_n8.rows")
+    for executor in ("0", "1"):
+        p = run(os.path.join(BIN, "allreduce"), "1053696", "stragglar", "2", "-1", "--schedule", rows, "--init", "uniform",
+                "--nocheck", "--report", "--executor", executor)
+        assert p.returncode == 0, p.stdout + p.stderr
+        assert ("executor=%s" % ("column" if executor == "1" else "rounds")) in p.stderr
+        assert "algorithmic_bytes=%d" % (4 * 1053696) in p.stderr
+    # without --nocheck the final comparison of the rank buffers fails, as it must: the rows are no AllReduce
+    p = run(os.path.join(BIN, "allreduce"), "1053696", "stragglar", "1", "-1", "--schedule", rows, "--init", "uniform")
+    assert p.returncode != 0 and "Rank buffers differ" in p.stdout
+
+
 @pytest.mark.parametrize("extra", [[], ["--executor", "0"], ["--forward", "0"], ["--alg", "ring", "--no-cpu"]])
 def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     """bench.py end to end (at 16 MiB per rank so that it takes a second): exactly one JSON line on stdout, the

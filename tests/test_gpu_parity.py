@@ -777,3 +777,42 @@ def test_spread_arena(gpu_ctx, sarlib, oracle):
     gpu_ctx.set_tuning(arena_spread=1)
     run_gpu(gpu_ctx, sarlib, "stragglar", n, small, dtype, read_golden("stragglar_n8_cu.txt"), tuning=dict(arena_spread=1))
     assert gpu_ctx.stats().arena_spread == 0
+
+
+def test_stream_probe(gpu_ctx, sarlib):
+    """sar_probe_streams, the yardstick kernel: every written stream ends as the fp32 sum of the job's read streams
+    (a constant pattern when nothing is read), in place where a rank is on both sides, whatever launch shape ran
+    last; ranges and alignment are checked on the host."""
+    import stragglar_amd as sa
+    n, elems = 8, 3 * 4096 + 8
+    ctx = gpu_ctx
+    ctx.alloc_ranks(n, elems * 4, "f32")
+    inputs = make_inputs(n, elems, "f32", seed=41, kind="ints")          # small integers: sums are exact in any order
+    for r, x in enumerate(inputs):
+        ctx.upload(r, x)
+    off, length = 16 * 5, 16 * 700                                       # bytes
+    lo, hi = off // 4, (off + length) // 4
+    res = ctx.probe_streams([([0, 1, 2], [3, 4], off), ([5, 6, 7], [5], off)], length, reps=1)
+    assert res.variants == 72 and res.best_ms > 0 and res.worst_ms >= res.best_ms and res.bytes_moved == (5 + 4) * length
+    assert res.block in (256, 512, 1024) and res.unroll in (1, 2, 4)
+    want = inputs[0][lo:hi] + inputs[1][lo:hi] + inputs[2][lo:hi]
+    for r in (3, 4):
+        got = ctx.download(r)
+        assert np.array_equal(got[lo:hi], want) and np.array_equal(got[:lo], inputs[r][:lo]) and np.array_equal(got[hi:], inputs[r][hi:])
+    # in place: rank 5 is read and written by every launch, 72 shapes x 2 launches each: s <- s + x6 + x7 every time
+    got = ctx.download(5)
+    assert np.array_equal(got[lo:hi], inputs[5][lo:hi] + 144 * (inputs[6][lo:hi] + inputs[7][lo:hi]))
+    for r in (0, 1, 2, 6, 7):
+        assert np.array_equal(ctx.download(r), inputs[r])
+    res = ctx.probe_streams([([], [0, 1], 0)], 16 * 64, reps=1)
+    assert res.variants == 36
+    assert np.array_equal(ctx.download(1)[:8], np.array([1, 2, 3, 4, 1, 2, 3, 4], np.float32))
+    for bad in ([([0], [1], 4)],                      # not on a 16-byte boundary
+                [([0], [8], 0)],                      # no such rank
+                [([0], [1], elems * 4)],              # leaves the buffer
+                [([0], [1], 0), ([0, 2], [3], 0)],    # jobs read different numbers of streams
+                [([], [], 0)]):
+        with pytest.raises(sa.SarError):
+            ctx.probe_streams(bad, 16 * 64, reps=1)
+    with pytest.raises(sa.SarError):
+        ctx.probe_streams([([0], [1], 0)], 24, reps=1)
