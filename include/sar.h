@@ -172,6 +172,11 @@ typedef struct sar_tuning_t {
                           /*     and so is a schedule that consists of such rows (the pre-work timed on its */
                           /*     own); 0 = they run in the multi-source kernel, one launch per round.       */
                           /*     Rows that are not whole 16-byte vectors on vector boundaries always do     */
+    int32_t col_depth_first; /* column executor, outside the plan for few work items: 1 = a work item takes a  */
+                          /*     row as soon as the values it consumes exist (a reduce tree is walked depth   */
+                          /*     first: log2 n values alive at a time instead of n/2, so fewer value slots    */
+                          /*     and more workgroups per compute unit); rows that touch a common chunk of a   */
+                          /*     rank keep their order, so the bits are the same; 0 = round order             */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */

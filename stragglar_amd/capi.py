@@ -77,7 +77,7 @@ class ProbeResult(ctypes.Structure):
 
 class Tuning(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd", "segments",
-                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "col_fuse_copies", "arena_spread", "col_prework")]
+                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "col_fuse_copies", "arena_spread", "col_prework", "col_depth_first")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

@@ -45,6 +45,7 @@ public:
         split_components();
         align_heads();
         choose_shape();
+        if (env_.tune.col_depth_first && !plan_.staged) order_depth_first();
         index_cells();
         Forwarding fwd = choose_forwarding();
         const Shape before = shape();
@@ -217,6 +218,83 @@ private:
             plan_.staged = true;
             plan_.block = lb;
         }
+    }
+
+    // The cells a row reads and writes.
+    void touches(const ColRow& r, std::vector<int>& reads, std::vector<int>& writes) const {
+        reads.clear(); writes.clear();
+        if (r.d.kind == SAR_OP_MREDUCE) { reads = r.mreads; writes = r.mwrites; return; }
+        reads.push_back(r.c1);
+        if (r.d.kind != SAR_OP_COPY) reads.push_back(r.c0);
+        writes.push_back(r.c0);
+        if (r.d.kind == SAR_OP_XREDUCE) writes.push_back(r.c1);
+        for (int cell : r.mwrites) writes.push_back(cell);
+    }
+
+    // Bandwidth plan: the order of a component's rows decides how many values are alive at a time, and with it the
+    // value slots a lane needs and the workgroups a compute unit holds.  Round order runs a reduce tree level by
+    // level (halving-doubling: n/2 partial sums alive after the first round); taking a row as soon as the values it
+    // consumes exist walks the tree depth first instead (log2 n alive: 3 slots instead of 4 at n = 8, 4 instead of
+    // 8 at n = 16).  Rows that touch a common cell, one of them writing it, keep their order; nothing else about a
+    // round is binding, since every lane meets only its own column.  Among the rows that may run next, one that
+    // reads a cell written by a row already placed goes first, else the earliest in round order.  Groups are cut
+    // anew: a row joins the open group unless it conflicts with a row in it.  Tables whose rows already come in
+    // this order (the StragglAR tables, ring, direct) are left as they are.
+    void order_depth_first() {
+        std::vector<ColRow> out; out.reserve(nrows());
+        std::vector<uint32_t> group_begin;
+        std::vector<ColumnComp> comps;
+        uint32_t max_groups = 0;
+        std::vector<int> rd, wr, rd2, wr2;
+        for (const auto& cc : plan_.comps) {
+            const uint32_t m = cc.row_end - cc.row_first;
+            // predecessors by conflict
+            std::vector<std::vector<uint32_t>> preds(m);
+            std::vector<std::vector<int>> reads(m), writes(m);
+            for (uint32_t j = 0; j < m; ++j) touches(cr_[cc.row_first + j], reads[j], writes[j]);
+            auto hits = [](const std::vector<int>& a, const std::vector<int>& b) {
+                for (int x : a) for (int y : b) if (x == y) return true;
+                return false;
+            };
+            for (uint32_t j = 0; j < m; ++j)
+                for (uint32_t i = 0; i < j; ++i)
+                    if (hits(writes[i], reads[j]) || hits(writes[i], writes[j]) || hits(reads[i], writes[j])) preds[j].push_back(i);
+            std::vector<char> placed(m, 0);
+            std::vector<uint32_t> order; order.reserve(m);
+            for (uint32_t step = 0; step < m; ++step) {
+                int pick = -1;
+                for (uint32_t j = 0; j < m && pick < 0; ++j) {          // a consumer of a value that exists already
+                    if (placed[j]) continue;
+                    bool ready = true, consumes = false;
+                    for (uint32_t i : preds[j]) { ready = ready && placed[i]; consumes = consumes || (placed[i] && hits(writes[i], reads[j])); }
+                    if (ready && consumes) pick = (int)j;
+                }
+                for (uint32_t j = 0; j < m && pick < 0; ++j) {          // else the earliest row whose turn it can be
+                    if (placed[j]) continue;
+                    bool ready = true;
+                    for (uint32_t i : preds[j]) ready = ready && placed[i];
+                    if (ready) pick = (int)j;
+                }
+                placed[(size_t)pick] = 1; order.push_back((uint32_t)pick);
+            }
+            ColumnComp nc{};
+            nc.group_first = (uint32_t)group_begin.size(); nc.row_first = (uint32_t)out.size();
+            uint32_t open = 0;                                          // first row (index into order) of the open group
+            for (uint32_t k = 0; k < m; ++k) {
+                bool conflict = k == 0;
+                for (uint32_t q = open; q < k && !conflict; ++q)
+                    conflict = std::find(preds[order[k]].begin(), preds[order[k]].end(), order[q]) != preds[order[k]].end() ||
+                               std::find(preds[order[q]].begin(), preds[order[q]].end(), order[k]) != preds[order[q]].end();
+                if (conflict) { group_begin.push_back((uint32_t)out.size()); open = k; }
+                out.push_back(cr_[cc.row_first + order[k]]);
+            }
+            nc.group_end = (uint32_t)group_begin.size(); nc.row_end = (uint32_t)out.size();
+            max_groups = std::max(max_groups, nc.group_end - nc.group_first);
+            comps.push_back(nc);
+        }
+        group_begin.push_back((uint32_t)out.size());
+        cr_.swap(out); plan_.group_begin.swap(group_begin); plan_.comps.swap(comps);
+        plan_.max_comp_groups = max_groups;
     }
 
     // per cell, the rows that touch it, in order

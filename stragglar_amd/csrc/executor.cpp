@@ -98,7 +98,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 0, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 0, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1};
 
     // prepared plan
     bool prepared = false;
@@ -636,7 +636,7 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
            (t.col_elide_stores == 0 || t.col_elide_stores == 1) && t.col_fuse_chains >= 0 && t.col_fuse_chains <= 2 && t.col_fuse_copies >= 0 && t.col_fuse_copies <= 2 &&
-           (t.arena_spread == 0 || t.arena_spread == 1) && (t.col_prework == 0 || t.col_prework == 1);
+           (t.arena_spread == 0 || t.arena_spread == 1) && (t.col_prework == 0 || t.col_prework == 1) && (t.col_depth_first == 0 || t.col_depth_first == 1);
 }
 
 // sar_plan / sar_plan_rows: a context that never touches the device, with the rank buffers at made-up, suitably

@@ -726,7 +726,8 @@ def test_random_row_lists(gpu_ctx, sarlib, oracle, seed):
               dict(executor=1, col_slots=2, col_elide_stores=0), dict(executor=1, col_latency_plan=0, col_slots=2),
               dict(executor=1, col_latency_plan=0, col_slots=8), dict(executor=1, col_latency_plan=2, col_slots=1, col_wgs=1),
               dict(executor=1, col_latency_plan=2, col_slots=5), dict(executor=1, col_latency_plan=0),
-              dict(executor=1, col_slots=4, col_light_sync=0, cache_policy=1, col_block=1024), dict(executor=2)):
+              dict(executor=1, col_slots=4, col_light_sync=0, cache_policy=1, col_block=1024), dict(executor=2),
+              dict(executor=1, col_latency_plan=0, col_depth_first=0, col_slots=2), dict(executor=1, col_latency_plan=0, col_split=0, col_slots=3)):
         ctx.set_tuning(**dict(ctx.default_tuning, **t))
         for r, x in enumerate(inputs):
             ctx.upload(r, x)

@@ -39,9 +39,12 @@ def test_stragglar_n8_plan(sarlib, table):
     assert st.col_slots == 1                                  # one value alive per item
     assert st.forwarded_bytes == 42 * C                       # every re-read
     assert st.col_block == 512
-    # all rows of a column in round order instead: four values alive at a time
-    st0 = plan(sarlib, "stragglar", 8, S, table=table, col_split=0)
+    # all rows of a column in round order instead: four values alive at a time; taking every row as soon as the
+    # value it consumes exists finishes one broadcast tree before the next exchange: one value alive again
+    st0 = plan(sarlib, "stragglar", 8, S, table=table, col_split=0, col_depth_first=0)
     assert st0.col_components == 1 and st0.col_slots == 4 and st0.forwarded_bytes == 42 * C
+    st1 = plan(sarlib, "stragglar", 8, S, table=table, col_split=0)
+    assert st1.col_components == 1 and st1.col_slots == 1 and st1.forwarded_bytes == 42 * C
     # forwarding off, one launch per round
     assert plan(sarlib, "stragglar", 8, S, table=table, col_forward=0).forwarded_bytes == 0
     st_r = plan(sarlib, "stragglar", 8, S, table=table, executor=0)
@@ -64,8 +67,14 @@ def test_comparators_n8_plan(sarlib):
     assert plan(sarlib, "ring", 8, S, col_forward=0).elided_store_bytes == 0
     rhd = plan(sarlib, "rhd", 8, S)
     assert rhd.algorithmic_bytes == 35 * S and rhd.rounds == 6
-    assert rhd.col_components == 8 and rhd.col_slots == 4     # a butterfly over 8 ranks: 4, 2, 1 partial sums alive
+    # a butterfly over 8 ranks, walked depth first: the sums of two pairs, their sum, the next two pairs ... three values
+    # alive at a time (log2 n); level by level, in round order, it is four (n / 2)
+    assert rhd.col_components == 8 and rhd.col_slots == 3
     assert rhd.forwarded_bytes == 8 * (6 + 7) * Cn            # reduce tree: 4 + 2 operands of the later steps; 7 copies
+    level = plan(sarlib, "rhd", 8, S, col_depth_first=0)
+    assert level.col_slots == 4 and level.forwarded_bytes == rhd.forwarded_bytes
+    assert plan(sarlib, "rhd", 16, sarlib.pad_bytes(256 * MIB, 16)).col_slots == 4
+    assert plan(sarlib, "rhd", 16, sarlib.pad_bytes(256 * MIB, 16), col_depth_first=0, col_block=256).col_slots == 8
     direct = plan(sarlib, "direct", 8, S)
     assert direct.algorithmic_bytes == 16 * S and direct.rounds == 3     # the exchange, then 2 + 4 copies
     assert direct.col_components == 1 and direct.col_slots == 1 and direct.forwarded_bytes == 6 * S
@@ -94,7 +103,8 @@ def test_small_messages_take_the_plan_for_few_items(sarlib):
     rhd = plan(sarlib, "rhd", 8, S)
     assert rhd.executor == 1 and rhd.col_slots == 4
     assert plan(sarlib, "rhd", 8, S, col_fuse_copies=0).col_slots == 0
-    assert plan(sarlib, "rhd", 8, S, col_latency_plan=0).col_slots == 4
+    assert plan(sarlib, "rhd", 8, S, col_latency_plan=0).col_slots == 3          # the bandwidth plan walks the tree depth first
+    assert plan(sarlib, "rhd", 8, S, col_latency_plan=0, col_depth_first=0).col_slots == 4
     rows, _ = sarlib.plan_rows(sarlib.builtin("rhd", 8), 8, S)
     assert len(rows) == 8 * 7 and all(r.kind == 2 for r in rows) and sum(r.ndst for r in rows) == 8 * 7
     # the four reduces of a chunk's first round load eight cold operands: they take them together (and the two of
@@ -289,7 +299,8 @@ def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
 
 PLAN_SETTINGS = [dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_slots=1), dict(col_latency_plan=0, col_slots=3, col_fuse_copies=2),
                  dict(col_latency_plan=2, col_slots=8), dict(col_forward=0), dict(col_split=0, col_slots=4), dict(col_latency_plan=0, col_elide_stores=0),
-                 dict(col_fuse_copies=0), dict(col_latency_plan=2, col_slots=2, col_fuse_copies=0, col_fuse_chains=0), dict(col_latency_plan=0, col_slots=8, col_fuse_copies=2)]
+                 dict(col_fuse_copies=0), dict(col_latency_plan=2, col_slots=2, col_fuse_copies=0, col_fuse_chains=0), dict(col_latency_plan=0, col_slots=8, col_fuse_copies=2),
+                 dict(col_latency_plan=0, col_depth_first=0), dict(col_latency_plan=0, col_depth_first=0, col_slots=3, col_fuse_copies=2), dict(col_latency_plan=0, col_split=0)]
 
 
 @pytest.mark.parametrize("dtype,chunk_elems", [("f32", 1024), ("f32", 4 * 37 + 1), ("bf16", 8 * 50), ("f16", 8 * 21 + 3)])
