@@ -23,6 +23,9 @@ algorithmic_GBps = the rows' algorithmic bytes / mean step time: every row
 roofline  = the same two figures for the dominant kernel (the column kernel:
             one launch per schedule; with --executor 0 the round kernel: one
             launch per round) from an event pair around every launch.
+stream_ceiling = what a kernel that only loads, adds and stores reaches for the
+            same streams on the same buffers (sar_probe_streams), live.
+reduce_steps_alone = the table's exchanges without its copies, same protocol.
 comparators = ring, rhd and direct on the same rank buffers and inputs.
 cpu_baseline = the CPU checker (oracle/, a port) executing the same schedule
             on the host cores of this box.
@@ -125,7 +128,7 @@ def main():
     ap.add_argument("--mib", type=int, default=256, help="unpadded MiB per rank")
     ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and the bit checks against the CPU checker")
-    ap.add_argument("--no-comparators", action="store_true", help="skip ring / rhd / direct on the same buffers")
+    ap.add_argument("--no-comparators", action="store_true", help="skip the legs beside the headline: ring / rhd / direct on the same buffers and the reduce steps alone")
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
     ap.add_argument("--executor", type=int, default=None, choices=[0, 1, 2],
                     help="0 = one launch per round, 1 = column executor (one launch per schedule), 2 = chosen by the library's cost model (default)")
@@ -270,6 +273,29 @@ def main():
                                  "shapes_tried": res.variants, "slowest_shape_ms": round(res.worst_ms, 5),
                                  "kernel_vs_ceiling": round(roofline["achieved"] / res.gbps, 4)}
         ctx.restore()
+
+    if args.alg == "stragglar" and not args.no_comparators:
+        # The reduce steps on their own: the n-1 exchanges of the table (round r: rank r and the straggler exchange
+        # chunk r and both add, allreduce_8GPU.cu:564-578 + reduce_add :29-34) as a schedule without the copies.  Two
+        # cold reads and two writes per element, in place: nothing to forward, so these bytes all reach memory.
+        rows = "sar-rows %d %d\n" % (n, n - 1) + "".join("round\nxreduce %d %d %d\n" % (r, n - 1, r) for r in range(n - 1))
+        xsched = lib.parse(rows, n)
+        ctx.prepare(xsched, None, use_graph=args.graph)
+        xst = ctx.stats()
+        xms = timed_steps(ctx, args.steps, args.warmup)
+        xm = statistics.fmean(xms)
+        xmem, xhbm, _ = rates(xst, xm)
+        rec["reduce_steps_alone"] = {"rows": "%d exchanges (XREDUCE) of one chunk each, no copies" % (n - 1), "ms_per_step": round(xm, 5),
+                                     "ms_per_step_min": round(min(xms), 5), "memory_bytes_per_step": int(xmem),
+                                     "GBps": round(xhbm, 1), "frac_of_hbm_peak": round(xhbm / HBM_PEAK_GBPS, 4),
+                                     "executor_used": "column" if xst.executor == 1 else "rounds", "launches": int(xst.launches)}
+        if 2 <= n - 1 <= 8:
+            chunk = (elems // (n - 1)) * 4
+            res = ctx.probe_streams([([r, n - 1], [r, n - 1], r * chunk) for r in range(n - 1)], chunk - chunk % 16, 5)
+            rec["reduce_steps_alone"]["stream_ceiling_GBps"] = round(res.gbps, 1)
+            rec["reduce_steps_alone"]["vs_ceiling"] = round(xhbm / res.gbps, 4)
+        ctx.restore()
+        ctx.prepare(main_sched, None, use_graph=False)
 
     orc = inputs = None
     if not args.no_cpu:

@@ -215,6 +215,8 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     assert abs(roof["achieved"] - roof["memory_bytes_per_launch"] / roof["mean_launch_ms"] / 1e6) <= 0.002 * roof["achieved"]
     assert rec["host"]["logical_cpus"] >= 1
     if "--alg" not in extra:
+        red = rec["reduce_steps_alone"]
+        assert red["memory_bytes_per_step"] == rec["algorithmic_bytes_per_step"] // 4 and red["GBps"] > 0       # 4 S of the 16 S
         assert sorted(rec["comparators"]) == ["direct", "rhd", "ring"]
         for leg in rec["comparators"].values():
             assert leg["ranks_identical_after_run"] is True and leg["ms_per_step"] > 0 and leg["memory_side_GBps"] > 0
