@@ -195,7 +195,7 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     // enough candidates to cross a region boundary from anywhere, no more
     const uint64_t budget = std::min<uint64_t>((uint64_t)free_b - kSpreadHeadroom, kSpreadSearch + 2 * bytes);
     std::vector<char*> held;
-    try { held.reserve((size_t)(budget / bytes) + 1); } catch (const std::bad_alloc&) { return SAR_SPREAD_NO_MEMORY; }      // no allocation below
+    try { held.reserve((size_t)(budget / bytes) + 2); } catch (const std::bad_alloc&) { return SAR_SPREAD_NO_MEMORY; }      // no allocation below
     // The first allocation, and the yardstick: the probe's time for two neighbouring windows at its start, which
     // share a region.  Should a boundary run through the allocation (its two ends then probe like a pair in
     // different regions), it stays held as a spacer and the one behind it takes its place.

@@ -395,6 +395,24 @@ def test_delay_mode(gpu_ctx, sarlib, oracle):
     assert ctx.sleep_ticks(5.0) > 0
 
 
+@pytest.mark.parametrize("col_prework", [1, 0])
+@pytest.mark.parametrize("alg,n", [("stragglar", 8), ("direct", 8), ("stragglar", 6), ("direct", 4), ("stragglar", 4)])
+def test_prework_beside_the_delay(gpu_ctx, sarlib, oracle, alg, n, col_prework):
+    """DELAY > 0 for both algorithms that have pre-work (stragglar_allreduce_delay :876-898 with its ReduceScatter,
+    direct_allreduce_delay :115-137 with its (n-1)-rank AllReduce), in the plan for few work items and in the
+    bandwidth plan, on whole-vector and on ragged sizes, with the pre-work as a column launch and in the
+    multi-source kernel: the same bits as with no delay."""
+    table = {8: "stragglar_n8_cu.txt", 6: "synth_nonpow2_n6.txt", 4: "stragglar_n4_cu.txt"}[n]
+    text = read_golden(table) if alg == "stragglar" else None
+    for dtype, elems in (("f32", sarlib.pad_bytes(64 << 10, n) // 4), ("bf16", sarlib.pad_bytes(6 << 20, n) // 2), ("f16", (n - 1) * 1531 + 3),
+                         ("f32", (n - 1) * 4 * 40000)):
+        inputs = make_inputs(n, elems, dtype, seed=elems % 97)
+        want = run_oracle(oracle, alg, inputs, dtype, text, delay=1.0)
+        got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=0.3, tuning=dict(col_prework=col_prework))
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "%s n=%d %s %d elements col_prework %d rank %d" % (alg, n, dtype, elems, col_prework, r))
+
+
 def test_reference_self_check_pattern(gpu_ctx, sarlib, oracle):
     """The reference's own check: constant fills end as 36.0 (n=8) / 6.0 (n=4) everywhere."""
     for n, base, expect in ((8, 1, 36.0), (4, 0, 6.0)):
