@@ -174,6 +174,17 @@ def test_measurement_tools_run():
     assert any(l.startswith("region of every group:") for l in lines)
 
 
+def test_size_sweep_tool():
+    import sys
+    p = run(sys.executable, "-m", "stragglar_amd.size_sweep", "--sizes", "4096,1048576", "--iters", "3")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = p.stdout.splitlines()
+    assert lines[0] == "algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps"
+    rows = [l.split(",") for l in lines[1:]]
+    assert len(rows) == 2 * 4 * 2 and {r[0] for r in rows} == {"stragglar", "ring", "rhd", "direct"}
+    assert {int(r[1]) for r in rows} == {7168, 1053696} and all(float(r[5]) >= float(r[6]) > 0 for r in rows)
+
+
 def test_cli_runs_a_row_list_that_is_no_allreduce():
     """--schedule with a row list, --nocheck, --executor: the exchanges of the n=8 table alone, both executors."""
     rows = os.path.join(ROOT, "stragglar_amd", "schedules", "exchanges_n8.rows")
