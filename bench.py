@@ -15,8 +15,8 @@ value     = bytes that reach memory per step / mean step time: an HBM rate,
             REDUCE_INTO 3 per payload byte) minus the operands the column
             kernel takes from LDS value slots instead of loading them again
             and minus the stores it leaves out because they are overwritten
-            unread.  The rocprofv3 counters (profiles/) measure the same
-            number within 0.01 %.
+            unread.  roofline.traffic is the same number by the hardware
+            counters, from two child runs of this script under rocprofv3 --pmc.
 algorithmic_GBps = the rows' algorithmic bytes / mean step time: every row
             priced on its own, whether or not its operand came from LDS.  It
             can pass the HBM peak and is not a roofline fraction.
@@ -102,6 +102,59 @@ def cpu_baseline(orc, inputs, n, elems, rounds, algorithmic_bytes, budget_s=25.0
     return out, bufs
 
 
+def live_traffic(args, kernel_pattern, bytes_per_rank):
+    """HBM bytes per launch of the dominant kernel by the hardware counters, measured now: two child runs of this
+    script under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
+    counter shows for a streaming kernel of known size in the same run (compare_kernel reads two rank buffers,
+    fill_random_kernel writes one).  None when the profiler is missing or a run fails: the caller then falls back to
+    the figure kept under profiles/."""
+    import csv
+    import glob
+    import re
+    import shutil
+    import subprocess
+    import tempfile
+    if not shutil.which("rocprofv3") or not shutil.which("timeout"):
+        return None
+    tmp = tempfile.mkdtemp(prefix="sar_traffic_")
+    env = dict(os.environ, TMPDIR=os.environ.get("TMPDIR", "/tmp"))
+    child = [sys.executable, os.path.join(ROOT, "bench.py"), "--no-cpu", "--no-comparators", "--traffic-child", "--steps", "3", "--warmup", "1",
+             "--ranks", str(args.ranks), "--mib", str(args.mib), "--alg", args.alg]
+    if args.executor is not None:
+        child += ["--executor", str(args.executor)]
+    if args.forward is not None:
+        child += ["--forward", str(args.forward)]
+    out = {}
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            d = os.path.join(tmp, counter)
+            cmd = ["timeout", "-s", "KILL", "120", "rocprofv3", "--pmc", counter, "--output-format", "csv", "-d", d, "--"] + child
+            p = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=150)
+            files = glob.glob(os.path.join(d, "*", "*_counter_collection.csv"))
+            if p.returncode != 0 or not files:
+                return None
+            per = {}
+            with open(files[0]) as f:
+                for row in csv.DictReader(f):
+                    per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+            def mean(pat):
+                v = [x for k, xs in per.items() if re.search(pat, k) for x in xs]
+                return sum(v) / len(v) if v else None
+            kib = bytes_per_rank / 1024.0
+            ref = mean("compare_kernel") if counter == "FETCH_SIZE" else mean("fill_random_kernel")
+            val = mean(kernel_pattern)
+            if not ref or val is None:
+                return None
+            out[counter] = (val, (2 * kib if counter == "FETCH_SIZE" else kib) / ref)
+    except Exception:
+        return None
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    (fetch, ff), (write, wf) = out["FETCH_SIZE"], out["WRITE_SIZE"]
+    return {"bytes": int(round((fetch * ff + write * wf) * 1024)), "fetch_kib": round(fetch, 1), "fetch_factor": round(ff, 5),
+            "write_kib": round(write, 1), "write_factor": round(wf, 5)}
+
+
 def timed_steps(ctx, steps, warmup):
     for _ in range(warmup):
         ctx.restore()
@@ -129,6 +182,8 @@ def main():
     ap.add_argument("--alg", default="stragglar", choices=["stragglar", "ring", "rhd", "direct"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and the bit checks against the CPU checker")
     ap.add_argument("--no-comparators", action="store_true", help="skip the legs beside the headline: ring / rhd / direct on the same buffers and the reduce steps alone")
+    ap.add_argument("--no-live-traffic", action="store_true", help="do not run the two rocprofv3 --pmc child runs that measure roofline.traffic; use the figure kept under profiles/")
+    ap.add_argument("--traffic-child", action="store_true", help=argparse.SUPPRESS)      # a run of this script under the profiler: headline steps only
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
     ap.add_argument("--executor", type=int, default=None, choices=[0, 1, 2],
                     help="0 = one launch per round, 1 = column executor (one launch per schedule), 2 = chosen by the library's cost model (default)")
@@ -164,6 +219,9 @@ def main():
 
     step_ms = timed_steps(ctx, args.steps, args.warmup)
     identical = ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts)
+    if args.traffic_child:
+        ctx.close()
+        return
     ms = statistics.fmean(step_ms)
     # the same K steps back to back on the host clock, no restore in between (the sums just keep growing):
     # a cross-check of the event timing that includes launch and synchronisation overhead
@@ -199,6 +257,17 @@ def main():
         if key in traffic_table:
             traffic = traffic_table[key]["hbm_bytes_per_launch"]
             traffic_source = "offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, %s (not measured by this run)" % traffic_table[key]["source"]
+    if not args.no_live_traffic and not args.traffic_child and not args.graph:
+        if st.executor == 1:
+            pattern = r"column_kernel<0, %d, %s," % (st.col_block, "true" if st.col_slots else "false")
+        else:
+            pattern = r"round_kernel<0,"
+        live = live_traffic(args, pattern, nbytes)
+        if live:
+            traffic = live["bytes"]
+            traffic_source = ("this run: two child runs under rocprofv3 --pmc (FETCH_SIZE %.1f KiB x %.5f + WRITE_SIZE %.1f KiB x %.5f per launch, "
+                              "factors from compare_kernel / fill_random_kernel of known size in the same runs)"
+                              % (live["fetch_kib"], live["fetch_factor"], live["write_kib"], live["write_factor"]))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "bytes": "bytes that reach memory per launch, from this run's plan: algorithmic - taken from LDS slots - stores left out",

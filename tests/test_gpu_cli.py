@@ -199,7 +199,7 @@ def test_cli_runs_a_row_list_that_is_no_allreduce():
     assert p.returncode != 0 and "Rank buffers differ" in p.stdout
 
 
-@pytest.mark.parametrize("extra", [[], ["--executor", "0"], ["--forward", "0"], ["--alg", "ring", "--no-cpu"]])
+@pytest.mark.parametrize("extra", [[], ["--executor", "0", "--no-live-traffic"], ["--forward", "0", "--no-live-traffic"], ["--alg", "ring", "--no-cpu", "--no-live-traffic"]])
 def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     """bench.py end to end (at 16 MiB per rank so that it takes a second): exactly one JSON line on stdout, the
     keys the harness reads, a roofline object and, for the StragglAR run, the CPU baseline."""
@@ -225,6 +225,13 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     assert rec["memory_bytes_per_step"] == rec["algorithmic_bytes_per_step"] - rec["forwarded_bytes_per_step"] - rec["elided_store_bytes_per_step"]
     assert abs(roof["achieved"] - roof["memory_bytes_per_launch"] / roof["mean_launch_ms"] / 1e6) <= 0.002 * roof["achieved"]
     assert rec["host"]["logical_cpus"] >= 1
+    if "--no-live-traffic" not in extra:
+        import shutil
+        if shutil.which("rocprofv3"):
+            # the counters of two child runs under the profiler, taken now: what reaches the fabric is what the plan says
+            # (at this size the rank buffers fit the Infinity Cache, which sits behind the counters)
+            assert roof["traffic_source"].startswith("this run"), roof["traffic_source"]
+            assert 0.98 <= roof["traffic_vs_plan"] <= 1.02, roof
     if "--alg" not in extra:
         red = rec["reduce_steps_alone"]
         assert red["memory_bytes_per_step"] == rec["algorithmic_bytes_per_step"] // 4 and red["GBps"] > 0       # 4 S of the 16 S
