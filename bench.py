@@ -200,19 +200,32 @@ def main():
     n, dtype = args.ranks, "f32"
     nbytes = lib.pad_bytes(args.mib << 20, n)
     elems = nbytes // 4
+    if args.alg == "stragglar":
+        main_sched, table_name = load_table(lib, n)
+    else:
+        main_sched, table_name = lib.builtin(args.alg, n), args.alg
+    overrides = {}
+    if args.executor is not None:
+        overrides["executor"] = args.executor
+    if args.forward is not None:
+        overrides["col_forward"] = args.forward
+    # The counters first, in child processes of their own, before this process touches the device: which kernel the
+    # schedule runs in is known from the plan, which needs no device.
+    live = None
+    if not args.no_live_traffic and not args.traffic_child and not args.graph:
+        pst = lib.plan(main_sched, n, nbytes, dtype, **overrides)
+        if pst.executor == 1:
+            pattern = r"column_kernel<0, %d, %s," % (pst.col_block, "true" if pst.col_slots else "false")
+        else:
+            pattern = r"round_kernel<0,"
+        live = live_traffic(args, pattern, nbytes)
     ctx = lib.context(0)              # raises without a usable device
     ctx.alloc_ranks(n, nbytes, dtype)
     for r in range(n):
         ctx.fill_uniform(r, 1000 + r, -1.0, 1.0)
     ctx.snapshot()
-    if args.alg == "stragglar":
-        main_sched, table_name = load_table(lib, n)
-    else:
-        main_sched, table_name = lib.builtin(args.alg, n), args.alg
-    if args.executor is not None:
-        ctx.set_tuning(executor=args.executor)
-    if args.forward is not None:
-        ctx.set_tuning(col_forward=args.forward)
+    if overrides:
+        ctx.set_tuning(**overrides)
     ctx.prepare(main_sched, None, use_graph=args.graph)
     st = ctx.stats()
     tune = ctx.get_tuning().as_dict()
@@ -257,17 +270,11 @@ def main():
         if key in traffic_table:
             traffic = traffic_table[key]["hbm_bytes_per_launch"]
             traffic_source = "offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, %s (not measured by this run)" % traffic_table[key]["source"]
-    if not args.no_live_traffic and not args.traffic_child and not args.graph:
-        if st.executor == 1:
-            pattern = r"column_kernel<0, %d, %s," % (st.col_block, "true" if st.col_slots else "false")
-        else:
-            pattern = r"round_kernel<0,"
-        live = live_traffic(args, pattern, nbytes)
-        if live:
-            traffic = live["bytes"]
-            traffic_source = ("this run: two child runs under rocprofv3 --pmc (FETCH_SIZE %.1f KiB x %.5f + WRITE_SIZE %.1f KiB x %.5f per launch, "
-                              "factors from compare_kernel / fill_random_kernel of known size in the same runs)"
-                              % (live["fetch_kib"], live["fetch_factor"], live["write_kib"], live["write_factor"]))
+    if live:
+        traffic = live["bytes"]
+        traffic_source = ("this run: two child runs under rocprofv3 --pmc (FETCH_SIZE %.1f KiB x %.5f + WRITE_SIZE %.1f KiB x %.5f per launch, "
+                          "factors from compare_kernel / fill_random_kernel of known size in the same runs)"
+                          % (live["fetch_kib"], live["fetch_factor"], live["write_kib"], live["write_factor"]))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "bytes": "bytes that reach memory per launch, from this run's plan: algorithmic - taken from LDS slots - stores left out",
