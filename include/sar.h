@@ -177,6 +177,9 @@ typedef struct sar_tuning_t {
                           /*     first: log2 n values alive at a time instead of n/2, so fewer value slots    */
                           /*     and more workgroups per compute unit); rows that touch a common chunk of a   */
                           /*     rank keep their order, so the bits are the same; 0 = round order             */
+    int32_t col_vectors;  /* column executor with value slots, outside the plan for few work items: 16-byte     */
+                          /*     vectors a lane moves per row, 1 or 2; 0 = chosen by the planner (two, except    */
+                          /*     for plans that mostly store, on payloads of 1 GiB and more)                     */
 } sar_tuning_t;
 
 /* ---- library ------------------------------------------------------- */
@@ -357,6 +360,9 @@ typedef struct sar_probe_result {
     int32_t block, unroll, nontemporal, persistent, interleave;      /* the fastest shape */
     int32_t variants;                 /* shapes tried */
     uint64_t bytes_moved;             /* (nread + nwrite) * bytes summed over the jobs */
+    float variant_ms[72];             /* every shape's time, in the order they are tried: threads 256, 512, 1024 (slowest     */
+                                      /* index) x vectors 1, 2, 4 x cached, streaming x tile per workgroup, resident grid x   */
+                                      /* jobs one after the other, taking turns (fastest index; one job: this level is absent) */
 } sar_probe_result;
 int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out);
 

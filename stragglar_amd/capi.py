@@ -68,7 +68,20 @@ class ProbeJob(ctypes.Structure):
 class ProbeResult(ctypes.Structure):
     _fields_ = [("best_ms", ctypes.c_float), ("worst_ms", ctypes.c_float), ("block", ctypes.c_int32), ("unroll", ctypes.c_int32),
                 ("nontemporal", ctypes.c_int32), ("persistent", ctypes.c_int32), ("interleave", ctypes.c_int32),
-                ("variants", ctypes.c_int32), ("bytes_moved", ctypes.c_uint64)]
+                ("variants", ctypes.c_int32), ("bytes_moved", ctypes.c_uint64), ("variant_ms", ctypes.c_float * 72)]
+
+    def shapes(self):
+        """(block, vectors per thread, streaming, resident grid, jobs take turns, ms) of every shape tried."""
+        out, k = [], 0
+        turns = (0, 1) if self.variants == 72 else (0,)
+        for block in (256, 512, 1024):
+            for unroll in (1, 2, 4):
+                for nt in (0, 1):
+                    for persistent in (0, 1):
+                        for il in turns:
+                            out.append((block, unroll, nt, persistent, il, self.variant_ms[k]))
+                            k += 1
+        return out
 
     @property
     def gbps(self) -> float:
@@ -77,7 +90,7 @@ class ProbeResult(ctypes.Structure):
 
 class Tuning(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("block", "unroll", "order", "cache_policy", "reuse_rounds", "reverse_odd", "segments",
-                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "col_fuse_copies", "arena_spread", "col_prework", "col_depth_first")]
+                                                 "executor", "col_wgs", "col_block", "col_forward", "col_slots", "col_light_sync", "col_latency_plan", "col_split", "col_fuse_prework", "col_elide_stores", "col_fuse_chains", "col_fuse_copies", "arena_spread", "col_prework", "col_depth_first", "col_vectors")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

@@ -66,6 +66,7 @@ public:
         plan_.nslots = fwd.nslots; plan_.forwarded_bytes = fwd.bytes;
         for (uint32_t i = 0; i < nrows(); ++i) { cr_[i].d.flags |= fwd.flags[i]; cr_[i].d.slots = fwd.slots[i]; }
         if (plan_.staged) mark_joins();
+        choose_vectors();
         choose_launch();
         for (const auto& r : cr_) { rows.push_back(r.d); plan_.multi_source |= r.d.kind == SAR_OP_MREDUCE; }
         return SAR_OK;
@@ -655,6 +656,31 @@ private:
         }
     }
 
+    // Vectors per lane and row where values are forwarded (bandwidth plan).  Two as a rule: what a row still loads
+    // is little and far between, and two loads in flight per lane pay (ring at 16 and 32 ranks: 4 to 5 %).  One for a
+    // plan that mostly stores -- the StragglAR tables and direct send two chunks' worth of cold reads and n chunks'
+    // worth of stores to memory -- once the payload is far beyond the Infinity Cache: more and smaller work items with
+    // streaming stores (see choose_launch) are the shape in which a kernel that does nothing else moves this mix
+    // fastest, and the schedule gains the same 2 to 3 % (n = 8, 256 MiB per rank: 416 -> 404 us; 1 GiB: 1658 -> 1628).
+    void choose_vectors() {
+        plan_.two_vectors = false; store_heavy_ = false;
+        if (!plan_.nslots || plan_.staged) return;
+        uint64_t reads = 0, writes = 0;
+        for (const auto& r : cr_) {
+            const DevOp& d = r.d;
+            const uint64_t b = d.bytes;
+            if (d.kind == SAR_OP_MREDUCE) { reads += b * d.nsrc; writes += (d.flags & DEVOP_DEAD0) ? 0 : b * d.ndst; continue; }
+            if (!(d.flags & DEVOP_GET1)) reads += b;
+            if (d.kind != SAR_OP_COPY && !(d.flags & DEVOP_GET0)) reads += b;
+            if (!(d.flags & DEVOP_DEAD0)) writes += b;
+            if (d.kind == SAR_OP_XREDUCE && !(d.flags & DEVOP_DEAD1)) writes += b;
+            writes += b * d.ndst;
+        }
+        store_heavy_ = all_found_ && writes >= 3 * reads && plan_.block >= 512 &&
+                       env_.bytes_per_rank * (uint64_t)env_.n >= (1ull << 30);
+        plan_.two_vectors = env_.tune.col_vectors ? env_.tune.col_vectors == 2 : !store_heavy_;
+    }
+
     void choose_launch() {
         // Cache policy of the launch (the column kernel takes one for all its rows).  Planned (2): when every re-read is
         // forwarded, what is still loaded is read exactly once: streaming loads (+1.5 % for the StragglAR table);
@@ -669,7 +695,9 @@ private:
         const int cp = env_.tune.cache_policy;
         bool only_multi_source = !cr_.empty();
         for (const auto& r : cr_) only_multi_source = only_multi_source && r.d.kind == SAR_OP_MREDUCE;
-        const uint32_t planned = all_found_ ? 1u : no_reuse_ ? (only_multi_source ? 2u : 1u) : 0u;
+        // A plan that mostly stores, one vector per lane, payload far beyond the Infinity Cache (choose_vectors): streaming
+        // stores as well, there is no use in keeping lines that nobody reads again.
+        const uint32_t planned = all_found_ ? (store_heavy_ && !plan_.two_vectors ? 2u : 1u) : no_reuse_ ? (only_multi_source ? 2u : 1u) : 0u;
         plan_.policy = cp == 0 ? 0u : cp == 1 ? 2u : cp == 3 ? 1u : planned;
 
         // Dispatch order of the items.  All columns of one component before the next component keeps the resident
@@ -688,7 +716,7 @@ private:
             }
             most = std::max(most, reducing);
         }
-        const uint64_t cbytes = column_bytes(plan_.block, plan_.nslots != 0 && !plan_.staged);
+        const uint64_t cbytes = plan_.column_bytes();
         const uint64_t items = (plan_.widest_row + cbytes - 1) / cbytes * plan_.comps.size();
         const uint64_t resident = (uint64_t)std::max(1, env_.compute_units) * (2048u / (uint32_t)plan_.block);
         plan_.component_major = most <= 1 && aligned && !plan_.staged && items >= 2 * resident;
@@ -711,6 +739,7 @@ private:
     std::vector<std::vector<Ev>> ev_;
     bool all_found_ = false;            // every re-read of a column finds its operand in a slot
     bool no_reuse_ = false;             // no row reads a cell that an earlier row read or wrote
+    bool store_heavy_ = false;          // every re-read forwarded, three times as many bytes stored as loaded, a large payload
 };
 
 }  // namespace

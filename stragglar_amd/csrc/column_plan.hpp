@@ -49,6 +49,8 @@ struct ColumnPlan {
     bool unsupported = false;        // the rows cannot all run in the column kernel
     bool multi_source = false;       // some rows are MREDUCE rows
     bool component_major = false;    // dispatch order of the items: all columns of a component, then the next component
+    bool two_vectors = false;        // with value slots, outside the latency plan: a lane moves two vectors per row (else one)
+    uint64_t column_bytes() const { return sar::column_bytes(block, two_vectors); }
 };
 
 // `scheds`: the schedules to run back to back in the one launch (the main schedule, or pre-work + main); they

@@ -72,7 +72,7 @@ struct ColumnDevice {
     bool ready = false;
     uint32_t* d_group_begin = nullptr;
     sar::ColumnComp* d_comps = nullptr;
-    uint32_t first_op = 0, ncomp = 0, ncols = 0, run = 1, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0, multi_source = 0;
+    uint32_t first_op = 0, ncomp = 0, ncols = 0, run = 1, items = 0, grid = 0, block = 512, slots = 0, lane_local = 0, table_rows = 0, table_groups = 0, policy = 0, multi_source = 0, two_vectors = 0;
 };
 
 struct sar_ctx {
@@ -98,7 +98,7 @@ struct sar_ctx {
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
-    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 0, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1};
+    sar_tuning_t tune{256, 1, 0, 2, 2, 0, 0, 2, 0, 0, 1, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0};
 
     // prepared plan
     bool prepared = false;
@@ -454,7 +454,7 @@ bool column_pays(const sar_ctx* c, const ColumnPlan& cp) {
         const double per_row_us = resident_bytes <= 262144.0 ? 0.32 : resident_bytes <= 33554432.0 ? 0.45 : 0.65;
         return 4.0 + std::max(item_rows * per_row_us, bytes / 5.5e6) <= est_rounds;
     }
-    const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
+    const uint64_t cb = cp.column_bytes();
     const double items = (double)((cp.widest_row + cb - 1) / cb) * (double)cp.comps.size();
     double wgs_per_cu = 2048.0 / cp.block;
     if (cp.nslots) wgs_per_cu = std::max(1.0, std::min(wgs_per_cu, std::floor(160.0 * 1024.0 / ((double)cp.nslots * (double)cb))));
@@ -477,7 +477,7 @@ int launch_column_plan(sar_ctx* c, const ColumnDevice& d, hipStream_t st) {
     L.ops = c->d_ops + d.first_op; L.group_begin = d.d_group_begin; L.comps = d.d_comps; L.ptrs = c->d_ptrs;
     L.ncomp = d.ncomp; L.nitems = d.items;
     L.table_rows = d.table_rows; L.table_groups = d.table_groups;
-    L.lane_local = d.lane_local; L.policy = d.policy; L.multi_source = d.multi_source;
+    L.lane_local = d.lane_local; L.policy = d.policy; L.multi_source = d.multi_source; L.two_vectors = d.two_vectors;
     L.ncols = d.ncols; L.run = d.run;
     SAR_HIP(sar::launch_column(c->dtype, (int)d.block, d.grid, d.slots, st, L));
     return SAR_OK;
@@ -486,7 +486,7 @@ int launch_column_plan(sar_ctx* c, const ColumnDevice& d) { return launch_column
 
 // Launch shape of a column plan whose rows sit in the row table from `first_op` on (no device work).
 int shape_column_plan(const sar_ctx* c, const ColumnPlan& cp, uint32_t first_op, ColumnDevice& d) {
-    const uint64_t cb = sar::column_bytes(cp.block, cp.nslots != 0 && !cp.staged);
+    const uint64_t cb = cp.column_bytes();
     const uint64_t ncols = (cp.widest_row + cb - 1) / cb;
     const uint64_t items = ncols * cp.comps.size();
     if (items > 0x7fffffffull) return set_error(SAR_EINVAL, "schedule needs more than 2^31 work items");
@@ -497,6 +497,7 @@ int shape_column_plan(const sar_ctx* c, const ColumnPlan& cp, uint32_t first_op,
     d.table_rows = cp.staged ? cp.max_comp_rows : 0u;
     d.table_groups = cp.staged ? cp.max_comp_groups + 1u : 0u;
     d.policy = cp.policy;
+    d.two_vectors = cp.two_vectors ? 1u : 0u;
     d.first_op = first_op; d.ncomp = (uint32_t)cp.comps.size(); d.ncols = (uint32_t)ncols;
     d.run = cp.component_major ? (uint32_t)ncols : 1u;        // d.run divides ncols either way: no padding items
     d.items = (uint32_t)items;
@@ -636,7 +637,7 @@ bool valid_tuning(const sar_tuning_t& t) {
            (t.col_light_sync == 0 || t.col_light_sync == 1) && t.col_latency_plan >= 0 && t.col_latency_plan <= 2 &&
            (t.col_split == 0 || t.col_split == 1) && (t.col_fuse_prework == 0 || t.col_fuse_prework == 1) &&
            (t.col_elide_stores == 0 || t.col_elide_stores == 1) && t.col_fuse_chains >= 0 && t.col_fuse_chains <= 2 && t.col_fuse_copies >= 0 && t.col_fuse_copies <= 2 &&
-           (t.arena_spread == 0 || t.arena_spread == 1) && (t.col_prework == 0 || t.col_prework == 1) && (t.col_depth_first == 0 || t.col_depth_first == 1);
+           (t.arena_spread == 0 || t.arena_spread == 1) && (t.col_prework == 0 || t.col_prework == 1) && (t.col_depth_first == 0 || t.col_depth_first == 1) && t.col_vectors >= 0 && t.col_vectors <= 2;
 }
 
 // sar_plan / sar_plan_rows: a context that never touches the device, with the rank buffers at made-up, suitably
@@ -1230,6 +1231,7 @@ static int probe_streams_body(sar_ctx* c, int njobs, const sar_probe_job* jobs, 
                             SAR_HIP(hipEventElapsedTime(&ms, c->ev_prof[0], c->ev_prof[1]));
                             if (r > 0 && (best < 0.f || ms < best)) best = ms;
                         }
+                        if (out->variants < 72) out->variant_ms[out->variants] = best;
                         out->variants += 1;
                         if (out->best_ms <= 0.f || best < out->best_ms) {
                             out->best_ms = best; out->block = block; out->unroll = unroll; out->nontemporal = nt;

@@ -494,14 +494,16 @@ __device__ __forceinline__ void lat_row_finish(const ColRow& row, uint64_t off, 
 // the two otherwise identical accesses are folded into one and the nontemporal hint is dropped.  MR: the
 // launch has multi-source rows (a pre-work collective in the same launch); their batched loads take more
 // registers and a longer row loop, so launches without such rows run a variant without that path.
-template <int DT, int BLOCK, bool FWD, bool LAT, int POL, bool MR>
+template <int DT, int BLOCK, bool FWD, bool LAT, int POL, bool MR, bool TWO>
 __global__ __launch_bounds__(BLOCK) void column_kernel(const DevOp* __restrict__ ops, const uint32_t* __restrict__ group_begin,
                                                         const ColumnComp* __restrict__ comps, char* const* __restrict__ ptrs, ColumnLaunch L) {
     typedef typename Elem<DT>::T T;
-    // Vectors per lane and row: two when values are forwarded in the bandwidth regime (the loads that remain are
-    // few and far between, and two in flight per lane pay: +2 to +9 %), one otherwise (every row loads and
-    // occupancy covers the latency; few items are better spread over more workgroups).
-    constexpr uint32_t V = (FWD && !LAT) ? 2u : 1u;
+    // Vectors per lane and row (TWO, only with FWD and without LAT): two when values are forwarded in the bandwidth
+    // regime and the rows still load a good part of their operands (the loads that remain are few and far between,
+    // and two in flight per lane pay: ring at 16 and 32 ranks +4 to +5 %), one otherwise: every row loads and
+    // occupancy covers the latency; few items are better spread over more workgroups; and a plan that mostly
+    // stores (the StragglAR tables, direct) runs 2 to 3 % faster with more, smaller work items.
+    constexpr uint32_t V = (FWD && !LAT && TWO) ? 2u : 1u;
     constexpr uint64_t col_bytes = (uint64_t)BLOCK * 16u * V;
     constexpr bool LNT = POL >= 1, SNT = POL == 2;
     // LDS: LAT: [the component's rows: table_rows x 64 B][its group boundaries: table_groups x 4 B, padded to
@@ -690,12 +692,12 @@ uint64_t column_lds_budget() { return 65536u; }
 uint64_t column_table_bytes(uint32_t rows, uint32_t groups) { return (uint64_t)rows * sizeof(DevOp) + (((uint64_t)groups + 3u) / 4u) * 16u; }
 int column_latency_block() { return 256; }
 
-template <int DT, bool FWD, int POL, bool MR>
+template <int DT, bool FWD, int POL, bool MR, bool TWO>
 static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hipStream_t st, const ColumnLaunch& L) {
     switch (block) {
-        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL, MR>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
-        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL, MR>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
-        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL, MR>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 256: hipLaunchKernelGGL((column_kernel<DT, 256, FWD, false, POL, MR, TWO>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 512: hipLaunchKernelGGL((column_kernel<DT, 512, FWD, false, POL, MR, TWO>), dim3(grid), dim3(512), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
+        case 1024: hipLaunchKernelGGL((column_kernel<DT, 1024, FWD, false, POL, MR, TWO>), dim3(grid), dim3(1024), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -704,11 +706,12 @@ static hipError_t launch_column_block(int block, uint32_t grid, uint32_t lds, hi
 template <int DT, int POL, bool MR>
 static hipError_t launch_column_policy(int block, uint32_t grid, uint32_t lds, bool fwd, hipStream_t st, const ColumnLaunch& L) {
     if (L.table_rows) {
-        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL, MR>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
-        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL, MR>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
+        if (fwd) hipLaunchKernelGGL((column_kernel<DT, 256, true, true, POL, MR, false>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
+        else hipLaunchKernelGGL((column_kernel<DT, 256, false, true, POL, MR, false>), dim3(grid), dim3(256), lds, st, L.ops, L.group_begin, L.comps, L.ptrs, L);
         return hipGetLastError();
     }
-    return fwd ? launch_column_block<DT, true, POL, MR>(block, grid, lds, st, L) : launch_column_block<DT, false, POL, MR>(block, grid, lds, st, L);
+    if (!fwd) return launch_column_block<DT, false, POL, MR, false>(block, grid, lds, st, L);
+    return L.two_vectors ? launch_column_block<DT, true, POL, MR, true>(block, grid, lds, st, L) : launch_column_block<DT, true, POL, MR, false>(block, grid, lds, st, L);
 }
 
 template <int DT>
@@ -724,7 +727,7 @@ static hipError_t launch_column_dt(int block, uint32_t grid, uint32_t lds, bool 
 hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, hipStream_t st, const ColumnLaunch& L) {
     if (L.nitems == 0 || grid == 0 || L.ncomp == 0) return hipSuccess;
     const bool lat = L.table_rows != 0;
-    const uint64_t lds = (lat ? column_table_bytes(L.table_rows, L.table_groups) : 0u) + (uint64_t)nslots * column_bytes(block, nslots != 0 && !lat);
+    const uint64_t lds = (lat ? column_table_bytes(L.table_rows, L.table_groups) : 0u) + (uint64_t)nslots * column_bytes(block, nslots != 0 && !lat && L.two_vectors);
     if (nslots > 255u || lds > column_lds_budget() || (lat && block != column_latency_block())) return hipErrorInvalidValue;
     switch (dtype) {
         case SAR_F32: return launch_column_dt<SAR_F32>(block, grid, (uint32_t)lds, nslots != 0, st, L);

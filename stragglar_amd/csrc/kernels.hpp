@@ -54,7 +54,7 @@ hipError_t launch_mreduce(int dtype, hipStream_t st, const DevOp* ops, uint32_t 
 // column executor: all rounds of COPY / REDUCE_INTO / XREDUCE rows (each exactly one chunk long) in one
 // launch.  The rows are sorted into components (sets of rows that share rank-chunk cells with each other and
 // with no other row); a work item is one component for one column of column_bytes(block, two_vectors) bytes: one
-// 16-byte vector per lane and row, two with forwarding (nslots > 0) outside the latency plan.
+// 16-byte vector per lane and row, or two (with forwarding, nslots > 0, outside the latency plan, where the plan says so).
 struct ColumnComp {
     uint32_t group_first, group_end;   // the component's groups (rows of one round each) in group_begin[]
     uint32_t row_first, row_end;       // = group_begin[group_first], group_begin[group_end]
@@ -73,6 +73,7 @@ struct ColumnLaunch {
     uint32_t lane_local;         // != 0 promises that no lane reads bytes another lane wrote (all rows 16-byte
                                  // aligned, no partial vectors): groups are then separated by an execution barrier only
     uint32_t policy;             // whole launch: 0 = cached accesses, 1 = streaming loads, 2 = streaming loads and stores
+    uint32_t two_vectors;        // with value slots and without a staged table: != 0 = a lane moves two 16-byte vectors per row
 };
 // With nslots > 0 a workgroup keeps up to nslots values per lane in LDS (nslots vectors per lane and vector of the row) and
 // rows flagged DEVOP_GET* take their operands from there instead of memory.  Slots plus the staged table

@@ -277,7 +277,9 @@ def test_value_forwarding_gives_the_same_bits(gpu_ctx, sarlib, oracle, alg, n, t
                   dict(col_forward=0, col_latency_plan=2, cache_policy=1),
                   dict(col_forward=1, col_split=0), dict(col_forward=0, col_split=0), dict(col_forward=1, col_split=0, col_latency_plan=2),
                   dict(col_forward=1, col_elide_stores=0), dict(col_forward=1, col_elide_stores=0, col_slots=2, col_latency_plan=2),
-                  dict(col_forward=1, col_fuse_chains=0, col_slots=2, col_latency_plan=2), dict(col_forward=1, col_slots=1, col_latency_plan=2, col_wgs=1)):
+                  dict(col_forward=1, col_fuse_chains=0, col_slots=2, col_latency_plan=2), dict(col_forward=1, col_slots=1, col_latency_plan=2, col_wgs=1),
+                  dict(col_forward=1, col_vectors=1), dict(col_forward=1, col_vectors=1, col_slots=3, col_block=1024), dict(col_forward=1, col_vectors=2, col_slots=2),
+                  dict(col_forward=1, col_vectors=1, col_elide_stores=0, cache_policy=1, col_light_sync=0), dict(col_forward=1, col_vectors=1, col_fuse_copies=2, col_block=256)):
             # these buffers have few columns: unless a case asks for it, keep the plan for few work items out of the way
             got = run_gpu(gpu_ctx, sarlib, alg, n, inputs, dtype, text, delay=-1.0, tuning=dict(dict(col_latency_plan=0), **dict(t, executor=1)))
             st = gpu_ctx.stats()
@@ -745,7 +747,9 @@ def test_random_row_lists(gpu_ctx, sarlib, oracle, seed):
               dict(executor=1, col_latency_plan=0, col_slots=8), dict(executor=1, col_latency_plan=2, col_slots=1, col_wgs=1),
               dict(executor=1, col_latency_plan=2, col_slots=5), dict(executor=1, col_latency_plan=0),
               dict(executor=1, col_slots=4, col_light_sync=0, cache_policy=1, col_block=1024), dict(executor=2),
-              dict(executor=1, col_latency_plan=0, col_depth_first=0, col_slots=2), dict(executor=1, col_latency_plan=0, col_split=0, col_slots=3)):
+              dict(executor=1, col_latency_plan=0, col_depth_first=0, col_slots=2), dict(executor=1, col_latency_plan=0, col_split=0, col_slots=3),
+              dict(executor=1, col_latency_plan=0, col_slots=3, col_vectors=1), dict(executor=1, col_latency_plan=0, col_vectors=1, col_block=512, cache_policy=1),
+              dict(executor=1, col_latency_plan=0, col_slots=2, col_vectors=2, col_block=1024)):
         ctx.set_tuning(**dict(ctx.default_tuning, **t))
         for r, x in enumerate(inputs):
             ctx.upload(r, x)

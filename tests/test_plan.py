@@ -300,7 +300,8 @@ def carry_out_plan(oracle, rows, ptrs, bufs, dtype):
 PLAN_SETTINGS = [dict(), dict(col_latency_plan=0), dict(col_latency_plan=0, col_slots=1), dict(col_latency_plan=0, col_slots=3, col_fuse_copies=2),
                  dict(col_latency_plan=2, col_slots=8), dict(col_forward=0), dict(col_split=0, col_slots=4), dict(col_latency_plan=0, col_elide_stores=0),
                  dict(col_fuse_copies=0), dict(col_latency_plan=2, col_slots=2, col_fuse_copies=0, col_fuse_chains=0), dict(col_latency_plan=0, col_slots=8, col_fuse_copies=2),
-                 dict(col_latency_plan=0, col_depth_first=0), dict(col_latency_plan=0, col_depth_first=0, col_slots=3, col_fuse_copies=2), dict(col_latency_plan=0, col_split=0)]
+                 dict(col_latency_plan=0, col_depth_first=0), dict(col_latency_plan=0, col_depth_first=0, col_slots=3, col_fuse_copies=2), dict(col_latency_plan=0, col_split=0),
+                 dict(col_latency_plan=0, col_vectors=1), dict(col_latency_plan=0, col_vectors=2, col_slots=2)]
 
 
 @pytest.mark.parametrize("dtype,chunk_elems", [("f32", 1024), ("f32", 4 * 37 + 1), ("bf16", 8 * 50), ("f16", 8 * 21 + 3)])
