@@ -103,6 +103,8 @@ typedef struct sar_stats_t {
     float spread_same_ms;          /* probed, the region probe's time for two windows in one region (the slowest  */
     float spread_pair_ms;          /* seen) and for the pair that was kept (the slower of its two probes), and    */
     uint64_t spread_search_bytes;  /* the most device memory held at a time while looking, the pair included      */
+    uint64_t fused_forwarded_bytes;    /* the same two figures for the single launch of pre-work + main schedule  */
+    uint64_t fused_elided_store_bytes; /* (fused_prework = 1), out of algorithmic_bytes + prework_bytes           */
 } sar_stats_t;
 
 /* run-time tunables of the executors; sar_get_tuning() reports the defaults */

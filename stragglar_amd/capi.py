@@ -44,7 +44,8 @@ class Stats(ctypes.Structure):
                 ("col_block", ctypes.c_int32), ("col_slots", ctypes.c_int32), ("col_components", ctypes.c_int32),
                 ("forwarded_bytes", ctypes.c_uint64), ("fused_prework", ctypes.c_int32), ("arena_spread", ctypes.c_int32),
                 ("elided_store_bytes", ctypes.c_uint64), ("spread_reason", ctypes.c_int32), ("spread_candidates", ctypes.c_int32),
-                ("spread_same_ms", ctypes.c_float), ("spread_pair_ms", ctypes.c_float), ("spread_search_bytes", ctypes.c_uint64)]
+                ("spread_same_ms", ctypes.c_float), ("spread_pair_ms", ctypes.c_float), ("spread_search_bytes", ctypes.c_uint64),
+                ("fused_forwarded_bytes", ctypes.c_uint64), ("fused_elided_store_bytes", ctypes.c_uint64)]
 
 
 class PlanRow(ctypes.Structure):

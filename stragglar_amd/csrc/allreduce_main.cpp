@@ -18,7 +18,8 @@
 //   --base B           constant of rank 0 for --init reference (default 1 for n=8, 0 for n=4, as the reference)
 //   --graph 0|1        replay the rounds as one hipGraph instead of launching them one by one (default 0:
 //                      on this software stack a replayed node costs more than an eager launch)
-//   --report           also print algorithmic GB/s and the HBM-roofline fraction to stderr
+//   --report           also print, to stderr, the bytes the timed part sends to memory, the rate and its fraction of
+//                      the 8 TB/s HBM peak, and the rows' algorithmic bytes and rate
 //   --executor 0|1|2   0 = one launch per round, 1 = the column kernel (one launch per schedule), 2 = the library's
 //                      choice (default)
 //   --nocheck          skip the final "all ranks hold the same" check: for a --schedule that times a part of a
@@ -212,13 +213,23 @@ int main(int argc, char* argv[]) {
         sum_ms += net; if (net < min_ms) min_ms = net;
     }
     if (report && numIters > 0) {
-        double total = (double)st.algorithmic_bytes + (sleepTime >= 0 ? (double)st.prework_bytes : 0.0);
+        // what the timed part of an iteration (runtime - delay) moves: the schedule, and the pre-work too when nobody is
+        // late (delay 0: it runs in front of the schedule; with a delay it runs beside the straggler's absence)
+        const bool with_prework = sleepTime == 0 && st.prework_bytes > 0;
+        const bool one_launch = with_prework && st.fused_prework;
+        const double algorithmic = (double)st.algorithmic_bytes + (with_prework ? (double)st.prework_bytes : 0.0);
+        const double on_chip = one_launch ? (double)st.fused_forwarded_bytes + (double)st.fused_elided_store_bytes
+                                          : (double)st.forwarded_bytes + (double)st.elided_store_bytes;
+        const double to_memory = algorithmic - on_chip;
         double mean = sum_ms / numIters;
-        fprintf(stderr, "# algorithmic_bytes=%.0f mean_ms=%.4f min_ms=%.4f algorithmic_GBps=%.1f (best %.1f) hbm_roofline_frac=%.3f launches=%d graph=%d\n",
-                total, mean, min_ms, total / mean / 1e6, total / min_ms / 1e6, total / mean / 1e6 / 8000.0, st.launches, st.uses_graph);
-        fprintf(stderr, "# executor=%s components=%d column_threads=%d value_slots=%d forwarded_bytes=%.0f elided_store_bytes=%.0f memory_side_GBps=%.1f prework_in_same_launch=%d ranks_in_two_hbm_regions=%d\n",
-                st.executor ? "column" : "rounds", st.col_components, st.col_block, st.col_slots, (double)st.forwarded_bytes, (double)st.elided_store_bytes,
-                (total - (double)st.forwarded_bytes - (double)st.elided_store_bytes) / mean / 1e6, (sleepTime == 0 && st.fused_prework) ? 1 : 0, st.arena_spread);
+        fprintf(stderr, "# bytes_to_memory=%.0f mean_ms=%.4f min_ms=%.4f memory_GBps=%.1f (best %.1f) frac_of_8TBps=%.3f algorithmic_bytes=%.0f algorithmic_GBps=%.1f launches=%d graph=%d\n",
+                to_memory, mean, min_ms, to_memory / mean / 1e6, to_memory / min_ms / 1e6, to_memory / mean / 1e6 / 8000.0, algorithmic, algorithmic / mean / 1e6,
+                one_launch ? 1 : st.launches - ((st.prework_bytes > 0 && !with_prework) ? 1 : 0), st.uses_graph);
+        fprintf(stderr, "# executor=%s components=%d column_threads=%d value_slots=%d taken_from_LDS_bytes=%.0f stores_left_out_bytes=%.0f prework=%s ranks_in_two_hbm_regions=%d\n",
+                st.executor ? "column" : "rounds", st.col_components, st.col_block, st.col_slots,
+                one_launch ? (double)st.fused_forwarded_bytes : (double)st.forwarded_bytes, one_launch ? (double)st.fused_elided_store_bytes : (double)st.elided_store_bytes,
+                one_launch ? "in the same launch" : with_prework ? "in front of the schedule" : st.prework_bytes > 0 ? "beside the delay (not in these figures)" : "none",
+                st.arena_spread);
     }
 
     // result check (allreduce_8GPU.cu:1069-1077 asserts 36.0; allreduce_4GPU.cu:593-603 prints mismatches)

@@ -604,7 +604,8 @@ int plan_on_host(sar_ctx* c, const sar_schedule* prework, const sar_schedule* ma
     return SAR_OK;
 }
 
-sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column, bool fused, bool pre_column) {
+sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_schedule* main_sched, const ColumnPlan& cp, bool column, bool fused, bool pre_column,
+                       const ColumnPlan* fp = nullptr) {
     sar_stats_t st{};
     sar::byte_counts(main_sched->s, c->elems(), elem_size_of(c->dtype), &st.algorithmic_bytes, &st.reference_op_bytes);
     if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
@@ -621,6 +622,7 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     st.forwarded_bytes = column ? cp.forwarded_bytes : 0;
     st.elided_store_bytes = column ? cp.elided_bytes : 0;
     st.fused_prework = fused ? 1 : 0;
+    if (fused && fp) { st.fused_forwarded_bytes = fp->forwarded_bytes; st.fused_elided_store_bytes = fp->elided_bytes; }
     st.arena_spread = c->spread() ? 1 : 0;
     st.spread_reason = c->spread_reason; st.spread_candidates = c->spread_candidates;
     st.spread_same_ms = c->spread_same_ms; st.spread_pair_ms = c->spread_pair_ms; st.spread_search_bytes = c->spread_search_bytes;
@@ -1072,7 +1074,7 @@ static int prepare_body(sar_ctx* c, const sar_schedule* prework, const sar_sched
     }
     if (hp.want_pre && (rc = upload_column_plan(c, hp.pp, hp.pre_first, c->pre)) != SAR_OK) { drop_plan(c); return rc; }
 
-    sar_stats_t st = plan_stats(c, prework, main_sched, hp.cp, c->column, c->fused.ready, c->pre.ready);
+    sar_stats_t st = plan_stats(c, prework, main_sched, hp.cp, c->column, c->fused.ready, c->pre.ready, &hp.fp);
     if (use_graph) {
         // the main rounds as one graph, and the single launch of pre-work + schedule (what sar_run with delay 0
         // runs) as another: kernel nodes only (no memset nodes)
@@ -1270,7 +1272,7 @@ static int plan_body(const sar_schedule* prework, const sar_schedule* main_sched
     HostPlan hp;
     const int rc = hp.make(prework, main_sched, n, bytes_per_rank, dtype, tuning, compute_units);
     if (rc != SAR_OK) return rc;
-    *out = plan_stats(&hp.c, prework, main_sched, hp.hp.cp, hp.hp.want_column, hp.hp.want_column && hp.hp.want_fused, hp.hp.want_pre);
+    *out = plan_stats(&hp.c, prework, main_sched, hp.hp.cp, hp.hp.want_column, hp.hp.want_column && hp.hp.want_fused, hp.hp.want_pre, &hp.hp.fp);
     return SAR_OK;
 }
 

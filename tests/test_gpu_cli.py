@@ -49,6 +49,16 @@ def test_delay_mode_prints_sleep_cycles_and_subtracts_delay():
     m = ROW.match(lines[2])
     assert m and m.group(4) == "2.000" and float(m.group(5)) >= 2.0
     assert "algorithmic_GBps" in p.stderr
+    # with a delay the pre-work runs beside it: the figures are the schedule's, 10 S to memory out of 16 S algorithmic
+    assert "bytes_to_memory=%d " % (10 * 1053696) in p.stderr and "algorithmic_bytes=%d " % (16 * 1053696) in p.stderr
+    assert "prework=beside the delay" in p.stderr
+    # nobody late: pre-work and schedule are one launch, 7 x 7 chunk reads for the pre-work + 7 for the exchanges, 56 chunk writes
+    p = run(os.path.join(BIN, "allreduce"), "1053696", "stragglar", "2", "0", "--report")
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "prework=in the same launch" in p.stderr and "launches=1 " in p.stderr
+    assert "bytes_to_memory=%d " % ((49 + 7 + 56) * 1053696 // 7) in p.stderr and "algorithmic_bytes=%d " % (24 * 1053696) in p.stderr
+    m = re.search(r"frac_of_8TBps=(\d+\.\d+)", p.stderr)
+    assert m and 0 < float(m.group(1)) < 1.0
 
 
 def test_other_dtypes_and_seeded_inputs():
