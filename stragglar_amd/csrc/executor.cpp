@@ -1416,21 +1416,28 @@ int run_static_body(int device, void* stream, const sar_schedule* prework, const
         return set_error(SAR_EINVAL, "the schedule's row tables take " + std::to_string(need) + " bytes, the static array of sar_run_static holds " +
                                          std::to_string((uint64_t)SAR_STATIC_SCRATCH_BYTES) + " (use sar_prepare / sar_run)");
     hipStream_t st = c.stream;
-    SAR_HIP(hipMemcpyAsync(base, rows.data() + lo, rows_b, hipMemcpyHostToDevice, st));
-    if (ptrs_b) SAR_HIP(hipMemcpyAsync(base + ptrs_at, ptrs.data(), ptrs_b, hipMemcpyHostToDevice, st));
     c.d_ops = (sar::DevOp*)base; c.d_ptrs = (char**)(base + ptrs_at);
     for (Launch& L : per_round) L.first_op -= (uint32_t)lo;
-    if ((rc = launch_all(&c, per_round, st)) != SAR_OK) { (void)hipStreamSynchronize(st); return rc; }
-    if (col) {
-        SAR_HIP(hipMemcpyAsync(base + grp_at, col->group_begin.data(), grp_b, hipMemcpyHostToDevice, st));
-        SAR_HIP(hipMemcpyAsync(base + comp_at, col->comps.data(), comp_b, hipMemcpyHostToDevice, st));
-        ColumnDevice d;
-        if ((rc = shape_column_plan(&c, *col, col_rows_first - (uint32_t)lo, d)) != SAR_OK) { (void)hipStreamSynchronize(st); return rc; }
-        d.d_group_begin = (uint32_t*)(base + grp_at); d.d_comps = (sar::ColumnComp*)(base + comp_at);
-        if ((rc = launch_column_plan(&c, d)) != SAR_OK) { (void)hipStreamSynchronize(st); return rc; }
-    }
-    // the result is complete, and the host copies of the tables are no longer needed, when the stream has drained
-    SAR_HIP(hipStreamSynchronize(st));
+    // Copies and launches on the caller's stream.  Whatever happens, the stream is drained before the host copies of
+    // the tables go out of scope; the result is complete when it has.
+    auto enqueue = [&]() -> int {
+        SAR_HIP(hipMemcpyAsync(base, rows.data() + lo, rows_b, hipMemcpyHostToDevice, st));
+        if (ptrs_b) SAR_HIP(hipMemcpyAsync(base + ptrs_at, ptrs.data(), ptrs_b, hipMemcpyHostToDevice, st));
+        int e = launch_all(&c, per_round, st); if (e) return e;
+        if (col) {
+            SAR_HIP(hipMemcpyAsync(base + grp_at, col->group_begin.data(), grp_b, hipMemcpyHostToDevice, st));
+            SAR_HIP(hipMemcpyAsync(base + comp_at, col->comps.data(), comp_b, hipMemcpyHostToDevice, st));
+            ColumnDevice d;
+            if ((e = shape_column_plan(&c, *col, col_rows_first - (uint32_t)lo, d)) != SAR_OK) return e;
+            d.d_group_begin = (uint32_t*)(base + grp_at); d.d_comps = (sar::ColumnComp*)(base + comp_at);
+            if ((e = launch_column_plan(&c, d)) != SAR_OK) return e;
+        }
+        return SAR_OK;
+    };
+    rc = enqueue();
+    const hipError_t drained = hipStreamSynchronize(st);
+    if (rc != SAR_OK) return rc;
+    if (drained != hipSuccess) return set_error(SAR_EHIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(drained));
     return SAR_OK;
 }
 
