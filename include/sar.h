@@ -56,7 +56,7 @@ enum {
     SAR_SPREAD_SMALL_PAYLOAD = 2,  /* less than 128 MiB over all ranks: the caches carry the schedule */
     SAR_SPREAD_UNKNOWN_DEVICE = 3, /* not a 288 GiB MI355X: the regions of this device are not known */
     SAR_SPREAD_NO_MEMORY = 4,      /* too little free device memory to look for a pair */
-    SAR_SPREAD_NO_PAIR = 5,        /* no candidate was faster against the first allocation than the first against itself */
+    SAR_SPREAD_NO_PAIR = 5,        /* no candidate was clearly faster against the first allocation than that is against itself */
     SAR_SPREAD_TOO_LARGE = 6,      /* half the ranks take more than 32 GiB */
     SAR_SPREAD_ADOPTED = 7         /* caller-owned buffers (sar_adopt_ranks) are taken where they are */
 };
@@ -100,8 +100,8 @@ typedef struct sar_stats_t {
                                    /* later row overwrites it and every reader in between takes it from a slot    */
     int32_t spread_reason;         /* SAR_SPREAD_*: why arena_spread is what it is                                */
     int32_t spread_candidates;     /* the search for the two allocations (last one this context ran): candidates  */
-    float spread_same_ms;          /* probed, the region probe's time for two windows in one region (the slowest  */
-    float spread_pair_ms;          /* seen) and for the pair that was kept (the slower of its two probes), and    */
+    float spread_same_ms;          /* probed, the region probe's time for two windows in one region (the fastest  */
+    float spread_pair_ms;          /* of four pairs) and for the pair that was kept (the slower of its two probes), and */
     uint64_t spread_search_bytes;  /* the most device memory held at a time while looking, the pair included      */
     uint64_t fused_forwarded_bytes;    /* the same two figures for the single launch of pre-work + main schedule  */
     uint64_t fused_elided_store_bytes; /* (fused_prework = 1), out of algorithmic_bytes + prework_bytes           */

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <stdexcept>
@@ -34,7 +35,10 @@ constexpr uint64_t kSpreadMinPayload = 128ull << 20;   // spread arena: from 16 
 constexpr uint64_t kSpreadHeadroom = 16ull << 30;      // memory left alone while looking for the pair
 constexpr uint64_t kSpreadMinAlloc = 8ull << 30, kSpreadMaxAlloc = 32ull << 30;      // per half; one size serves most payloads
 constexpr uint64_t kSpreadSearch = 96ull << 30;        // candidates held while looking, beyond the pair itself: one region
-constexpr float kSpreadFaster = 0.93f;                 // a pair in different regions takes at most this fraction of a pair in one
+constexpr float kSpreadFaster = 0.94f;                 // a pair in different regions takes at most this fraction of the fastest pair within one
+                                                       // (measured 0.87 to 0.895; candidates in the same region 1.0 and more)
+constexpr float kSpreadStraddle = 0.86f;               // the two ends of an allocation against its neighbouring windows: below this a boundary runs through it
+                                                       // (measured 0.80 with a boundary, 0.90 to 0.93 without)
 constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 streams of this size (beyond what the Infinity Cache absorbs)
 constexpr float kMaxDelayMs = 60000.f;
 
@@ -178,17 +182,17 @@ float probe_ms(sar_ctx* c, char* a, char* b, int reps) {
 // which region a buffer falls in is all that matters, not where in it.  Where an allocation lands physically is
 // the driver's business, so candidates are allocated one after the other and each is timed against the first
 // with a short probe (eight write streams of 128 MiB, four in either allocation) until one turns out to lie
-// elsewhere; the others are given back.  The yardstick is the probe's own time for two windows that do share a
-// region -- two neighbouring windows of the first allocation --, not a fixed figure: elsewhere means at most
-// kSpreadFaster of that, twice, on different windows of both (measured: 154-162 us against 175-212 us for
-// candidates in the first allocation's region, 181 us for its own two windows).  At most one region's worth of
-// candidates is held at a time beyond the pair.  Nothing is assumed about the order in which the driver hands
-// out memory, and a wrong verdict costs speed, not correctness: without a pair the caller falls back to one
-// allocation.  Returns a SAR_SPREAD_* reason.
+// elsewhere; the others are given back.  The yardstick is the probe's own time for windows that do share a
+// region, not a fixed figure: the fastest of four pairs of windows of the first allocation (three neighbouring
+// pairs and its two ends; measured 181-213 us, candidates in the same region 183-217 us, elsewhere 158-162 us).
+// Elsewhere means at most kSpreadFaster of that fastest pair, twice, on different windows of both.  At most one
+// region's worth of candidates is held at a time beyond the pair.  Nothing is assumed about the order in which
+// the driver hands out memory, and a wrong verdict costs speed, not correctness: without a pair the caller falls
+// back to one allocation.  Returns a SAR_SPREAD_* reason.
 int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     const uint64_t window = 4 * kProbeStream;
     c->spread_candidates = 0; c->spread_same_ms = c->spread_pair_ms = 0.f; c->spread_search_bytes = 0;
-    if (bytes < 2 * window) return SAR_SPREAD_NO_PAIR;
+    if (bytes < 8 * window) return SAR_SPREAD_NO_PAIR;
     size_t free_b = 0, total_b = 0;
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); return SAR_SPREAD_NO_MEMORY; }
     if (free_b < 4 * bytes + kSpreadHeadroom) return SAR_SPREAD_NO_MEMORY;
@@ -196,18 +200,25 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     const uint64_t budget = std::min<uint64_t>((uint64_t)free_b - kSpreadHeadroom, kSpreadSearch + 2 * bytes);
     std::vector<char*> held;
     try { held.reserve((size_t)(budget / bytes) + 2); } catch (const std::bad_alloc&) { return SAR_SPREAD_NO_MEMORY; }      // no allocation below
-    // The first allocation, and the yardstick: the probe's time for two neighbouring windows at its start, which
-    // share a region.  Should a boundary run through the allocation (its two ends then probe like a pair in
-    // different regions), it stays held as a spacer and the one behind it takes its place.
+    const bool debug = std::getenv("SAR_DEBUG_SPREAD") != nullptr;
+    // The first allocation and the yardstick.  Should a region boundary run through the allocation, its two ends
+    // probe like a pair in different regions while its neighbouring windows do not (ends at most kSpreadStraddle of
+    // the median neighbouring pair; without a boundary the ends take 0.90 to 0.93 of it): the allocation then stays
+    // held as a spacer and the one behind it takes its place.
     char* lo = nullptr;
     float same = -1.f;
     uint64_t used = 0;
     for (int attempt = 0; attempt < 2 && used + bytes <= budget; ++attempt) {
         if (hipMalloc((void**)&lo, bytes) != hipSuccess) { (void)hipGetLastError(); lo = nullptr; break; }
         used += bytes;
-        same = probe_ms(c, lo, lo + window, 3);
+        float adj[3];
+        for (int k = 0; k < 3; ++k) adj[k] = probe_ms(c, lo + (uint64_t)(2 * k) * window, lo + (uint64_t)(2 * k + 1) * window, 3);
         const float ends = probe_ms(c, lo, lo + bytes - window, 3);
-        if (same > 0.f && ends > 0.f && ends < kSpreadFaster * same && attempt == 0) { held.push_back(lo); lo = nullptr; continue; }
+        if (adj[0] <= 0.f || adj[1] <= 0.f || adj[2] <= 0.f || ends <= 0.f) { same = -1.f; break; }
+        std::sort(adj, adj + 3);
+        if (debug) std::fprintf(stderr, "sar spread: first allocation %p, neighbouring windows %.1f %.1f %.1f us, ends %.1f us\n", (void*)lo, adj[0] * 1e3, adj[1] * 1e3, adj[2] * 1e3, ends * 1e3);
+        if (ends < kSpreadStraddle * adj[1] && attempt == 0) { held.push_back(lo); lo = nullptr; continue; }
+        same = std::min(ends, adj[0]);
         break;
     }
     char* hi = nullptr;
@@ -216,9 +227,11 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
         if (hipMalloc((void**)&cand, bytes) != hipSuccess) { (void)hipGetLastError(); break; }
         c->spread_candidates += 1;
         const float t = probe_ms(c, lo, cand, 3);
+        if (debug) std::fprintf(stderr, "sar spread: candidate %d %p %.1f us (limit %.1f us)\n", c->spread_candidates, (void*)cand, t * 1e3, kSpreadFaster * same * 1e3);
         if (t < 0.f) { (void)hipFree(cand); break; }
         if (t < kSpreadFaster * same) {
             const float t2 = probe_ms(c, lo + bytes - window, cand + bytes - window, 3);
+            if (debug) std::fprintf(stderr, "sar spread: candidate %d, other windows %.1f us\n", c->spread_candidates, t2 * 1e3);
             if (t2 > 0.f && t2 < kSpreadFaster * same) { hi = cand; c->spread_pair_ms = std::max(t, t2); used += bytes; break; }
         }
         held.push_back(cand);

@@ -20,6 +20,11 @@ from __future__ import annotations
 import os
 from typing import List, Optional, Sequence
 
+# torch comes first on purpose.  It ships its own copy of the HIP runtime under the soname this package's library
+# asks for: with torch loaded first that copy serves both; with the library loaded first the process ends up with
+# two runtimes and the one initialised second reports "no ROCm-capable device is detected".
+import torch  # noqa: F401
+
 from . import capi
 
 _HERE = os.path.dirname(os.path.abspath(__file__))

@@ -215,7 +215,9 @@ def test_rank_tensors_are_placed_by_the_library(oracle):
             inputs = [to_np_bits(t).copy() for t in tensors]
             group.all_reduce(tensors)
             st = group._ctx.stats()
-            assert st.spread_reason in (0, 3) and st.arena_spread == (1 if st.spread_reason == 0 else 0)      # 3: not a 288 GiB device
+            why = "reason %d, %d candidates, probe %.1f us within a region, %.1f us for the pair, %.1f GiB held" % (
+                st.spread_reason, st.spread_candidates, st.spread_same_ms * 1e3, st.spread_pair_ms * 1e3, st.spread_search_bytes / 2.0 ** 30)
+            assert st.spread_reason in (0, 3) and st.arena_spread == (1 if st.spread_reason == 0 else 0), why      # 3: not a 288 GiB device
             order = list(range(n))
             order[6], order[7] = order[7], order[6]
             want = [inputs[i].copy() for i in order]
@@ -224,3 +226,38 @@ def test_rank_tensors_are_placed_by_the_library(oracle):
                 assert_bits_equal(to_np_bits(tensors[i]), want[k], "%s rank %d" % (name, i))
     finally:
         group.close()
+
+
+def test_data_parallel_step_through_dist_all_reduce(c10d_group):
+    """The reference trainer's gradient exchange (dp.py:28-65: flatten the gradients, dist.all_reduce(SUM), divide by
+    the world size, copy back) with eight replicas of a small model emulated on one GPU: the flat gradient buffers are the
+    rows of one tensor, padded as example.py:19 pads, and after the step every replica holds the mean gradient."""
+    import torch.distributed as dist
+    n = 8
+    torch.manual_seed(0)
+    proto = torch.nn.Sequential(torch.nn.Linear(37, 64), torch.nn.Tanh(), torch.nn.Linear(64, 11)).cuda()
+    replicas = []
+    for r in range(n):
+        m = torch.nn.Sequential(torch.nn.Linear(37, 64), torch.nn.Tanh(), torch.nn.Linear(64, 11)).cuda()
+        m.load_state_dict(proto.state_dict())
+        x = torch.randn(16, 37, device="cuda", generator=torch.Generator(device="cuda").manual_seed(100 + r))
+        m(x).square().mean().backward()
+        replicas.append(m)
+    grads = [[p.grad for p in m.parameters()] for m in replicas]
+    numel = sum(g.numel() for g in grads[0])
+    padded = c10d_group.padded_numel(numel, n, 4)
+    flat = torch.zeros(n, padded, device="cuda")                       # flatten_tensors (dp.py:28-39), one row per replica
+    for r in range(n):
+        flat[r, :numel] = torch.cat([g.reshape(-1) for g in grads[r]])
+    want = flat[:, :numel].double().sum(dim=0) / n
+    dist.all_reduce(flat, op=dist.ReduceOp.SUM)                        # dp.py:59
+    flat /= n                                                          # dp.py:60
+    for r in range(n):                                                 # unflatten_tensors + copy back (dp.py:41-65)
+        off = 0
+        for g in grads[r]:
+            g.copy_(flat[r, off:off + g.numel()].view_as(g))
+            off += g.numel()
+    for r in range(n):
+        got = torch.cat([p.grad.reshape(-1) for p in replicas[r].parameters()]).double()
+        assert torch.allclose(got, want, rtol=1e-6, atol=1e-9), "replica %d" % r
+        assert torch.equal(flat[r], flat[0])                           # every replica holds the same bits
