@@ -327,7 +327,9 @@ int sar_run(sar_ctx* ctx, float delay_ms, float* elapsed_ms);
  * GPU, held until the process ends; a schedule whose tables need more is refused with SAR_EINVAL (the n = 8
  * tables take a few KiB, a 64-rank ring about half a MiB).  `stream` is the caller's hipStream_t (NULL = the
  * null stream): the tables are copied and the kernels launched on it, and the call returns when it has drained
- * and the result is complete.  device_ptrs as for sar_adopt_ranks (checked the same way); the default tuning
+ * and the result is complete (so `stream` itself must not be capturing: the call is for a process that has a
+ * capture open elsewhere, or may not allocate for other reasons; the table copies are hipMemcpyAsync from
+ * ordinary host memory, staged by the runtime).  device_ptrs as for sar_adopt_ranks (checked the same way); the default tuning
  * applies.  No context is needed or touched.  All calls on one GPU share the one array, which keeps the last
  * call's tables: calls that overlap in time on the same GPU race and must be serialised by the caller. */
 int sar_run_static(int device, void* stream, const sar_schedule* prework, const sar_schedule* main_sched, int n,

@@ -678,7 +678,11 @@ private:
         }
         store_heavy_ = all_found_ && writes >= 3 * reads && plan_.block >= 512 &&
                        env_.bytes_per_rank * (uint64_t)env_.n >= (1ull << 30);
-        plan_.two_vectors = env_.tune.col_vectors ? env_.tune.col_vectors == 2 : !store_heavy_;
+        // Three value slots and more (halving-doubling) on payloads of 1 GiB and more: the slots of two vectors per lane are what limits the workgroups
+        // resident on a compute unit, and one vector per lane runs level or ahead (n = 8, 1 GiB per rank: 2816 -> 2763 us;
+        // n = 32 and 64, 2 GiB over all ranks: -2 and -3 %; n = 8 and 16 at 2 GiB: level).
+        const bool slot_bound = plan_.nslots >= 3 && env_.bytes_per_rank * (uint64_t)env_.n >= (1ull << 30);
+        plan_.two_vectors = env_.tune.col_vectors ? env_.tune.col_vectors == 2 : !store_heavy_ && !slot_bound;
     }
 
     void choose_launch() {
