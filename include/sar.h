@@ -370,6 +370,18 @@ typedef struct sar_probe_result {
 } sar_probe_result;
 int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out);
 
+/* The two decisions sar_alloc_ranks takes when it looks for a second allocation in another region of HBM (tuning
+ * arena_spread), as functions of the region probe's times alone -- no device is touched; tests feed them recorded
+ * times.  No counterpart in the reference (one buffer per GPU: allreduce_8GPU.cu:977-990).
+ * sar_spread_yardstick: neighbours_ms = the probe's time for three pairs of neighbouring windows of the first
+ * allocation, ends_ms = for its first and last window.  *yardstick_ms = the fastest of the four, the time of a pair
+ * that shares a region.  Returns 0, or 1 when the ends are so much faster than the median neighbouring pair that a
+ * region boundary must run through the allocation (the search then sets it aside and starts from the next one).
+ * sar_spread_is_elsewhere: 1 when a candidate's probe time against the first allocation says "another region"
+ * (clearly below the yardstick), else 0.  Negative = SAR_EINVAL. */
+int sar_spread_yardstick(const float* neighbours_ms, float ends_ms, float* yardstick_ms);
+int sar_spread_is_elsewhere(float yardstick_ms, float probe_ms);
+
 /* Ticks of the device's constant-rate wall clock that delay_ms lasts: the
  * figure the CLI prints as "Sleep cycles" (calculate_sleep_cycles,
  * allreduce_8GPU.cu:47-58, uses ms * clockRate_kHz of the shader clock). */

@@ -117,6 +117,7 @@ EXPORTS = [
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
     "sar_run_static", "sar_static_scratch_bytes", "sar_rank_pointer", "sar_probe_streams",
+    "sar_spread_yardstick", "sar_spread_is_elsewhere",
 ]
 
 
@@ -175,6 +176,8 @@ class Library:
             "sar_static_scratch_bytes": (u64, []),
             "sar_rank_pointer": (c_int, [vp, c_int, P(vp)]),
             "sar_probe_streams": (c_int, [vp, c_int, P(ProbeJob), u64, c_int, P(ProbeResult)]),
+            "sar_spread_yardstick": (c_int, [P(ctypes.c_float), ctypes.c_float, P(ctypes.c_float)]),
+            "sar_spread_is_elsewhere": (c_int, [ctypes.c_float, ctypes.c_float]),
         }
         assert sorted(sig) == sorted(EXPORTS)
         for name, (res, args) in sig.items():
@@ -193,6 +196,22 @@ class Library:
 
     def pad_bytes(self, nbytes: int, n: int) -> int:
         return int(self.lib.sar_pad_bytes(nbytes, n))
+
+    def spread_yardstick(self, neighbours_ms, ends_ms: float):
+        """(yardstick in ms, whether a region boundary runs through the first allocation) from the region probe's
+        times for three neighbouring pairs of its windows and for its two ends."""
+        arr = (ctypes.c_float * 3)(*neighbours_ms)
+        y = ctypes.c_float(0.0)
+        rc = self.lib.sar_spread_yardstick(arr, ends_ms, ctypes.byref(y))
+        if rc < 0:
+            self.check(rc)
+        return y.value, bool(rc)
+
+    def spread_is_elsewhere(self, yardstick_ms: float, probe_ms: float) -> bool:
+        rc = self.lib.sar_spread_is_elsewhere(yardstick_ms, probe_ms)
+        if rc < 0:
+            self.check(rc)
+        return bool(rc)
 
     def default_tuning(self) -> "Tuning":
         t = Tuning()

@@ -176,6 +176,18 @@ float probe_ms(sar_ctx* c, char* a, char* b, int reps) {
     return best;
 }
 
+// The two decisions of the region search as functions of probe times alone, so that they can be checked against
+// recorded times without a device (sar_spread_yardstick, sar_spread_is_elsewhere).
+// Yardstick: the fastest of the four pairs of windows within the first allocation.  Returns false when the
+// allocation's two ends probe like different regions against its median neighbouring pair: a boundary runs through it.
+bool spread_yardstick(const float neighbours_ms[3], float ends_ms, float* yardstick_ms) {
+    float adj[3] = {neighbours_ms[0], neighbours_ms[1], neighbours_ms[2]};
+    std::sort(adj, adj + 3);
+    *yardstick_ms = std::min(ends_ms, adj[0]);
+    return !(ends_ms < kSpreadStraddle * adj[1]);
+}
+bool spread_is_elsewhere(float yardstick_ms, float probe_ms_value) { return probe_ms_value > 0.f && probe_ms_value < kSpreadFaster * yardstick_ms; }
+
 // Two allocations of `bytes` each that lie in different regions of HBM.  Measured on MI355X: the 288 GiB behave as
 // three regions of 96 GiB (presumably the stack levels of the 12-high HBM3E), and streams that run at the same
 // time in different regions get in each other's way less: the write-heavy schedules here gain 15 to 25 %, and
@@ -215,10 +227,9 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
         for (int k = 0; k < 3; ++k) adj[k] = probe_ms(c, lo + (uint64_t)(2 * k) * window, lo + (uint64_t)(2 * k + 1) * window, 3);
         const float ends = probe_ms(c, lo, lo + bytes - window, 3);
         if (adj[0] <= 0.f || adj[1] <= 0.f || adj[2] <= 0.f || ends <= 0.f) { same = -1.f; break; }
-        std::sort(adj, adj + 3);
         if (debug) std::fprintf(stderr, "sar spread: first allocation %p, neighbouring windows %.1f %.1f %.1f us, ends %.1f us\n", (void*)lo, adj[0] * 1e3, adj[1] * 1e3, adj[2] * 1e3, ends * 1e3);
-        if (ends < kSpreadStraddle * adj[1] && attempt == 0) { held.push_back(lo); lo = nullptr; continue; }
-        same = std::min(ends, adj[0]);
+        const bool whole = spread_yardstick(adj, ends, &same);
+        if (!whole && attempt == 0) { held.push_back(lo); lo = nullptr; same = -1.f; continue; }
         break;
     }
     char* hi = nullptr;
@@ -229,10 +240,10 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
         const float t = probe_ms(c, lo, cand, 3);
         if (debug) std::fprintf(stderr, "sar spread: candidate %d %p %.1f us (limit %.1f us)\n", c->spread_candidates, (void*)cand, t * 1e3, kSpreadFaster * same * 1e3);
         if (t < 0.f) { (void)hipFree(cand); break; }
-        if (t < kSpreadFaster * same) {
+        if (spread_is_elsewhere(same, t)) {
             const float t2 = probe_ms(c, lo + bytes - window, cand + bytes - window, 3);
             if (debug) std::fprintf(stderr, "sar spread: candidate %d, other windows %.1f us\n", c->spread_candidates, t2 * 1e3);
-            if (t2 > 0.f && t2 < kSpreadFaster * same) { hi = cand; c->spread_pair_ms = std::max(t, t2); used += bytes; break; }
+            if (spread_is_elsewhere(same, t2)) { hi = cand; c->spread_pair_ms = std::max(t, t2); used += bytes; break; }
         }
         held.push_back(cand);
     }
@@ -1255,6 +1266,17 @@ static int probe_streams_body(sar_ctx* c, int njobs, const sar_probe_job* jobs, 
                         if (best > out->worst_ms) out->worst_ms = best;
                     }
     return SAR_OK;
+}
+
+int sar_spread_yardstick(const float* neighbours_ms, float ends_ms, float* yardstick_ms) {
+    if (!neighbours_ms || !yardstick_ms) return set_error(SAR_EINVAL, "null argument");
+    if (!(neighbours_ms[0] > 0.f && neighbours_ms[1] > 0.f && neighbours_ms[2] > 0.f && ends_ms > 0.f)) return set_error(SAR_EINVAL, "probe times must be positive");
+    return spread_yardstick(neighbours_ms, ends_ms, yardstick_ms) ? 0 : 1;
+}
+
+int sar_spread_is_elsewhere(float yardstick_ms, float probe_ms_value) {
+    if (!(yardstick_ms > 0.f)) return set_error(SAR_EINVAL, "the yardstick must be positive");
+    return spread_is_elsewhere(yardstick_ms, probe_ms_value) ? 1 : 0;
 }
 
 int sar_probe_streams(sar_ctx* c, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out) {

@@ -500,3 +500,44 @@ def test_rows_that_share_a_cell_do_not_take_their_operands_together(sarlib):
         fills_in_run = {q.put_slot for q in second[run_start:k] if q.put_slot >= 0}
         assert not (r.joins and ({r.get0_slot, r.get1_slot} & fills_in_run)), (k, fills)
     assert any(r.joins for r in second)
+
+
+# Region probe times recorded on MI355X boxes (microseconds): per search the three neighbouring pairs of windows of the
+# first allocation, its two ends, the times of candidates that share its region and of the pair that lay elsewhere
+# (first probe, second probe on other windows).
+_RECORDED_SEARCHES = [
+    ((180.8, 205.7, 198.9), 185.2, (185.5, 190.4, 212.0, 197.7, 201.3), (160.4, 158.5)),
+    ((202.0, 204.5, 200.1), 181.5, (182.8, 184.9, 190.0, 195.1), (158.3, 159.3)),
+    ((211.9, 199.7, 203.0), 184.7, (206.0, 189.2, 190.3), (160.1, 158.9)),
+    ((195.5, 196.3, 198.3), 186.9, (183.4, 199.0), (158.5, 158.0)),
+    ((192.7, 194.5, 209.1), 184.5, (216.9, 187.2), (161.0, 163.5)),
+    ((200.8, 202.1, 202.2), 189.1, (193.3,), (165.4, 163.8)),
+    ((198.0, 200.2, 202.1), 186.9, (), (162.8, 162.8)),
+]
+
+
+def test_region_search_decisions_on_recorded_probe_times(sarlib):
+    """The yardstick is the fastest pair of windows within the first allocation; a candidate lies elsewhere only when it is
+    clearly faster than that.  An earlier form compared against ONE neighbouring pair (up to 213 us) and took candidates of
+    the same region at 183-190 us for another region: those must be turned down, and an allocation whose ends are merely
+    the fastest of its own pairs must not be mistaken for one with a boundary in it."""
+    for neighbours, ends, same_region, elsewhere in _RECORDED_SEARCHES:
+        y, straddles = sarlib.spread_yardstick([t * 1e-3 for t in neighbours], ends * 1e-3)
+        assert not straddles, (neighbours, ends)
+        assert abs(y * 1e3 - min(min(neighbours), ends)) < 1e-3
+        for t in same_region:
+            assert not sarlib.spread_is_elsewhere(y, t * 1e-3), (neighbours, ends, t)
+        for t in elsewhere:
+            assert sarlib.spread_is_elsewhere(y, t * 1e-3), (neighbours, ends, t)
+    # a boundary inside the first allocation: its ends probe like a pair in two regions, its neighbouring windows do not
+    y, straddles = sarlib.spread_yardstick([0.199, 0.203, 0.160], 0.159)
+    assert straddles
+    # ... and with such a yardstick nothing would pass, so the search sets the allocation aside instead of using it
+    assert not sarlib.spread_is_elsewhere(y, 0.159)
+    # failed probes (negative) and nonsense never count as elsewhere; bad arguments are refused
+    assert not sarlib.spread_is_elsewhere(0.185, -1.0)
+    assert not sarlib.spread_is_elsewhere(0.185, 0.0)
+    with pytest.raises(Exception):
+        sarlib.spread_yardstick([0.2, 0.0, 0.2], 0.18)
+    with pytest.raises(Exception):
+        sarlib.spread_is_elsewhere(0.0, 0.1)
