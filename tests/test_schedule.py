@@ -311,3 +311,47 @@ def test_shipped_schedules_are_current(sarlib):
         if n & (n - 1) == 0 or pytest.importorskip("networkx"):
             assert text == table_text(gen_schedules.synthesize(n))
         assert sarlib.parse(text, n).validate() == ""
+
+
+_C_CALLER = r"""
+#include "sar.h"
+#include <stdio.h>
+#include <string.h>
+int main(void) {
+    sar_schedule* s = 0;
+    sar_schedule* none = 0;
+    char msg[256];
+    sar_tuning_t t;
+    sar_stats_t st;
+    if (sar_schedule_builtin("ring", 8, &s) != SAR_OK) return 1;
+    if (sar_schedule_validate(s, msg, sizeof msg) != SAR_OK) return 2;
+    if (sar_default_tuning(&t) != SAR_OK) return 3;
+    memset(&st, 0, sizeof st);
+    if (sar_plan(0, s, 8, 268441600ull, SAR_F32, &t, 256, &st) != SAR_OK) return 4;
+    if (sar_schedule_builtin("no such algorithm", 8, &none) == SAR_OK || none) return 5;
+    printf("%llu %d %d %s\n", (unsigned long long)sar_pad_bytes(268435456ull, 8), sar_schedule_rounds(s), (int)st.executor, sar_last_error());
+    sar_schedule_free(s);
+    return 0;
+}
+"""
+
+
+def test_a_plain_c_program_uses_the_header_and_the_library(tmp_path):
+    """include/sar.h is C (C99, no warnings under -pedantic) and a C caller links against the shared library: what a
+    binding in any language with a C FFI relies on.  Host-only entry points; no device is touched."""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.join(root, "stragglar_amd", "lib")
+    if not os.path.exists(os.path.join(libdir, "libsar_hip.so")):
+        pytest.skip("library not built")
+    src = tmp_path / "caller.c"
+    src.write_text(_C_CALLER)
+    exe = tmp_path / "caller"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"), str(src),
+                    "-L", libdir, "-lsar_hip", "-Wl,-rpath," + libdir, "-o", str(exe)], check=True, capture_output=True, text=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 3)
+    assert out[0] == "268441600" and out[1] == "14" and out[2] == "1"
+    assert "no such algorithm" in out[3] or "unknown" in out[3].lower()
