@@ -215,7 +215,7 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     keys the harness reads, a roofline object and, for the StragglAR run, the CPU baseline."""
     import json
     import sys
-    p = run(sys.executable, os.path.join(ROOT, "bench.py"), "--mib", "16", "--steps", "3", "--warmup", "1", *extra)
+    p = run(sys.executable, os.path.join(ROOT, "bench.py"), "--mib", "16", "--steps", "3", "--warmup", "1", "--cpu-seconds", "0.3", *extra)
     assert p.returncode == 0, p.stdout + p.stderr
     lines = [l for l in p.stdout.splitlines() if l.strip()]
     assert len(lines) == 1, p.stdout
