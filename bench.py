@@ -118,6 +118,10 @@ def live_traffic(args, kernel_pattern, bytes_per_rank):
     import tempfile
     if not shutil.which("rocprofv3") or not shutil.which("timeout"):
         return None
+    # already under a profiler (its tool library is preloaded into this process and would be into the children):
+    # no profiler inside a profiler
+    if "rocprof" in os.environ.get("LD_PRELOAD", "").lower() or any(k.startswith(("ROCPROF", "ROCP_TOOL")) for k in os.environ):
+        return None
     tmp = tempfile.mkdtemp(prefix="sar_traffic_")
     env = dict(os.environ, TMPDIR=os.environ.get("TMPDIR", "/tmp"))
     child = [sys.executable, os.path.join(ROOT, "bench.py"), "--no-cpu", "--no-comparators", "--traffic-child", "--steps", "3", "--warmup", "1",
