@@ -632,6 +632,19 @@ def test_config5_1gib_fp32_all_algorithms(gpu_ctx, sarlib, oracle, executor):
     full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor, nbytes, seed=5000)
 
 
+@pytest.mark.parametrize("executor", [0, 1])
+def test_rank_buffers_beyond_4gib(gpu_ctx, sarlib, oracle, executor):
+    """Byte offsets within a rank buffer that do not fit 32 bits: n=8, 5 GiB fp32 per rank (40 GiB resident plus the
+    snapshot), the four algorithms, both executors.  The last two of the seven StragglAR chunks, the upper three of
+    ring's eight and the upper fifth of direct's whole-buffer rows lie beyond 4 GiB."""
+    nbytes = sarlib.pad_bytes(5 << 30, 8)
+    assert nbytes > 1 << 32
+    try:
+        full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor, nbytes, seed=7000)
+    finally:
+        gpu_ctx.alloc_ranks(2, 4096, "f32")      # give the 80 GiB back before the next test
+
+
 def test_config3_bf16_1gib_with_delay(gpu_ctx, sarlib, oracle):
     """Benchmark configuration 3: n=8 x 1 GiB bf16 (padded 1 073 744 896 B), normal(0, 1e-3) seeded per rank,
     sums accumulated in bf16, straggler rank 7 late by DELAY = 5 ms while ranks 0-6 reduce-scatter."""
