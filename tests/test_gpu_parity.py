@@ -806,7 +806,7 @@ def test_spread_arena(gpu_ctx, sarlib, oracle):
     print(why)
     if st.spread_reason != 3:                    # 3: not a 288 GiB device, regions unknown
         assert seen[0] == 1 and st.spread_reason == 0, why
-        assert 0 < st.spread_pair_ms < 0.92 * st.spread_same_ms, why          # measured 0.87 to 0.895; a pair in one region: 1.0 and more
+        assert 0 < st.spread_pair_ms < 0.94 * st.spread_same_ms, why          # the search's own limit; measured 0.87 to 0.895, a pair in one region 1.0 and more
         assert st.spread_search_bytes <= (96 + 2 * 8 + 1) << 30, why
     # small payloads stay back to back
     small = make_inputs(n, 7 * 8 * 100, dtype, seed=78)
