@@ -84,6 +84,7 @@ class EmulatedGroup:
         if reason:
             raise ValueError("invalid schedule: " + reason)
         self._key = None
+        self._placed = None            # ((numel, dtype), tensors) of the last rank_tensors call while its memory is in use
 
     def close(self):
         self._ctx.close()
@@ -92,13 +93,17 @@ class EmulatedGroup:
         """One flat tensor of ``numel`` elements per emulated rank, in memory the library allocates and places
         itself (``sar_alloc_ranks``: from 128 MiB over all ranks, half the ranks in another region of HBM than the
         rest, which is worth 15 to 25 % of the bandwidth and which tensors that torch allocated next to each other
-        cannot have).  The tensors alias the group's memory: they are valid until the next ``rank_tensors`` call or
-        ``close``.  ``all_reduce`` on them skips the adoption step."""
+        cannot have).  The tensors alias the group's memory: they are valid until a ``rank_tensors`` call for another
+        size or dtype, an ``all_reduce`` on tensors of the caller's own, or ``close``; a call for the same size and
+        dtype returns the same tensors.  ``all_reduce`` on them skips the adoption step."""
         import torch
         name = _TORCH_DTYPES.get(str(dtype))
         if name is None:
             raise TypeError("unsupported dtype %s" % dtype)
         es = capi.ELEM_SIZE[name]
+        if self._placed is not None and self._placed[0] == (numel, name):
+            return list(self._placed[1])               # the same buffers again: nothing to allocate or lower
+        self._placed = None
         self._ctx.alloc_ranks(self.n, numel * es, name)
         order = list(range(self.n))
         order[self.straggler], order[self.n - 1] = order[self.n - 1], order[self.straggler]
@@ -112,6 +117,7 @@ class EmulatedGroup:
             out[i] = t.view(torch.bfloat16) if name == "bf16" else t
         self._ctx.prepare(self._main, self._prework)
         self._key = (tuple(ptrs), numel * es, name)
+        self._placed = ((numel, name), tuple(out))
         return out
 
     def _order(self, tensors):
@@ -144,6 +150,7 @@ class EmulatedGroup:
         nbytes = t0.numel() * t0.element_size()
         key = (tuple(t.data_ptr() for t in ordered), nbytes, dtype)
         if key != self._key:                       # new buffers: adopt them and lower the schedule onto them
+            self._placed = None                    # (the library's own rank memory goes when other buffers are adopted)
             self._ctx.adopt_ranks(list(key[0]), nbytes, dtype)
             self._ctx.prepare(self._main, self._prework)
             self._key = key
@@ -152,20 +159,25 @@ class EmulatedGroup:
 
     def allreduce_gradients(self, per_rank_grads: Sequence[Sequence], average: bool = True):
         """dp.py:28-65 for all emulated ranks at once: flatten each rank's gradient tensors into one padded
-        buffer, AllReduce, divide by the world size, copy back into the gradient tensors."""
+        buffer, AllReduce, divide by the world size, copy back into the gradient tensors.  The flat buffers are
+        ``rank_tensors`` of the padded size (kept between steps of the same size); they are returned."""
         import torch
         if len(per_rank_grads) != self.n:
             raise ValueError("need one gradient list per emulated rank")
         parts = self._main.parts
-        flats = []
-        for grads in per_rank_grads:
-            flat = torch.cat([g.reshape(-1) for g in grads])
-            # padded as example.py:19 pads: chunks of whole KiB, so that every chunk is a whole number of 16-byte
-            # vectors on a vector boundary (the rows then run as vectors, pre-work and schedule as one launch)
-            pad = padded_numel(flat.numel(), self.n, flat.element_size(), parts) - flat.numel()
-            if pad:
-                flat = torch.cat([flat, flat.new_zeros(pad)])
-            flats.append(flat.contiguous())
+        first = per_rank_grads[0]
+        numel = sum(g.numel() for g in first)
+        # padded as example.py:19 pads: chunks of whole KiB, so that every chunk is a whole number of 16-byte
+        # vectors on a vector boundary (the rows then run as vectors, pre-work and schedule as one launch)
+        padded = padded_numel(numel, self.n, first[0].element_size(), parts)
+        # the flat buffers are the library's own rank memory (placed in two regions of HBM, kept from step to step)
+        flats = self.rank_tensors(padded, first[0].dtype)
+        for grads, flat in zip(per_rank_grads, flats):
+            if sum(g.numel() for g in grads) != numel or any(g.dtype != first[0].dtype for g in grads):
+                raise ValueError("every rank needs the same gradient sizes and dtype")
+            torch.cat([g.reshape(-1) for g in grads], out=flat[:numel])
+            if padded > numel:
+                flat[numel:].zero_()
         self.all_reduce(flats)
         for grads, flat in zip(per_rank_grads, flats):
             if average:

@@ -76,16 +76,34 @@ def test_gradient_averaging_like_the_reference_trainer():
     n = 4
     shapes = [(33, 7), (129,), (5, 5, 5)]
     g = torch.Generator(device="cpu").manual_seed(3)
-    grads = [[torch.randn(s, generator=g).cuda() for s in shapes] for _ in range(n)]
-    expect = [sum(grads[r][k].double() for r in range(n)) / n for k in range(len(shapes))]
     group = EmulatedGroup(n)
     try:
+        flats = None
+        for step in range(3):                      # the flat buffers are the library's and stay from step to step
+            grads = [[torch.randn(s, generator=g).cuda() for s in shapes] for _ in range(n)]
+            expect = [sum(grads[r][k].double() for r in range(n)) / n for k in range(len(shapes))]
+            again = group.allreduce_gradients(grads)
+            assert flats is None or [t.data_ptr() for t in again] == [t.data_ptr() for t in flats]
+            flats = again
+            for r in range(n):
+                for k in range(len(shapes)):
+                    assert torch.allclose(grads[r][k].double(), expect[k], rtol=0, atol=1e-6)
+        # another size, then tensors of the caller's own, then gradients again
+        other = [[torch.randn(1000, generator=g).cuda().half()] for _ in range(n)]
+        expect = sum(o[0].double() for o in other) / n
+        group.allreduce_gradients(other)
+        assert torch.allclose(other[2][0].double(), expect, rtol=0, atol=2e-3)
+        mine = [torch.full((3 * 1024,), float(r), device="cuda") for r in range(n)]
+        group.all_reduce(mine)
+        assert all(torch.all(t == 6.0) for t in mine)
+        grads = [[torch.randn(s, generator=g).cuda() for s in shapes] for _ in range(n)]
+        expect = [sum(grads[r][k].double() for r in range(n)) / n for k in range(len(shapes))]
         group.allreduce_gradients(grads)
+        for r in range(n):
+            for k in range(len(shapes)):
+                assert torch.allclose(grads[r][k].double(), expect[k], rtol=0, atol=1e-6)
     finally:
         group.close()
-    for r in range(n):
-        for k in range(len(shapes)):
-            assert torch.allclose(grads[r][k].double(), expect[k], rtol=0, atol=1e-6)
 
 
 def test_adopt_rejects_bad_buffers(sarlib):
