@@ -274,6 +274,19 @@ int sar_adopt_ranks(sar_ctx* ctx, int n, void* const* device_ptrs, uint64_t byte
  * kernels on the rank buffers or hand them on; valid until the ranks are allocated or adopted anew. */
 int sar_rank_pointer(sar_ctx* ctx, int rank, void** device_ptr);
 
+/* n rows of bytes_per_row bytes back to back in ONE virtual address range, row r at *base + r * bytes_per_row: memory
+ * for a caller that keeps the emulated ranks as the rows of one [n, numel] tensor, as the one-process counterpart of
+ * the reference's backend does (the tensor handed to dist.all_reduce, implementation/custom_backend/example.py:21-29),
+ * and then passes the row addresses to sar_adopt_ranks.  With the tuning's arena_spread on, a 288 GiB device and 128 MiB
+ * or more in all, rows [0, ceil(n/2)) and the rest lie in two physical allocations that were found to sit in
+ * different regions of HBM (the search sar_alloc_ranks uses) and are mapped next to each other, which rows of an
+ * ordinary allocation cannot have; *placed says whether (may be null), *reason why not (SAR_SPREAD_*, may be null).
+ * Otherwise a plain allocation.  The rows belong to the context: valid until the next sar_alloc_rows, sar_free_rows
+ * or sar_destroy; rank buffers adopted from them are dropped with them.  A placed pair (2 x 8 GiB, more for larger
+ * halves) stays with the context after sar_free_rows for the next call. */
+int sar_alloc_rows(sar_ctx* ctx, int n, uint64_t bytes_per_row, void** base, int* placed, int* reason);
+int sar_free_rows(sar_ctx* ctx);
+
 int sar_upload(sar_ctx* ctx, int rank, uint64_t byte_off, const void* host, uint64_t bytes);
 int sar_download(sar_ctx* ctx, int rank, uint64_t byte_off, void* host, uint64_t bytes);
 

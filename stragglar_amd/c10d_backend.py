@@ -129,9 +129,27 @@ class EmulatedProcessGroup(dist.ProcessGroup):
         self._groups.clear()
 
 
+_created = []          # weak references to the process groups made here, the newest last
+
+
 def create_backend(store, rank, size, timeout):
     """createBackendDummy (dummy.cpp:813-819): store and timeout are not used."""
-    return EmulatedProcessGroup(rank, size)
+    import weakref
+    pg = EmulatedProcessGroup(rank, size)
+    _created.append(weakref.ref(pg))
+    return pg
+
+
+def empty_ranks(n: int, numel: int, dtype=torch.float32):
+    """An uninitialised ``[n, numel]`` tensor for ``dist.all_reduce`` in memory the newest process group of this backend
+    allocates through the library (``EmulatedGroup.rank_block``): an ordinary contiguous tensor whose two halves lie
+    in different regions of HBM from 128 MiB in all, which a ``torch.empty`` cannot have (15 to 25 % of the bandwidth
+    at large sizes).  One such tensor per rank count at a time; it lives as long as the process group."""
+    for ref in reversed(_created):
+        pg = ref()
+        if pg is not None:
+            return pg._group(n).rank_block(numel, dtype)
+    raise RuntimeError("no process group of the %r backend: call dist.init_process_group first" % BACKEND_NAME)
 
 
 def register():

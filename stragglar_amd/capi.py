@@ -117,7 +117,7 @@ EXPORTS = [
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
     "sar_run_static", "sar_static_scratch_bytes", "sar_rank_pointer", "sar_probe_streams",
-    "sar_spread_yardstick", "sar_spread_is_elsewhere",
+    "sar_spread_yardstick", "sar_spread_is_elsewhere", "sar_alloc_rows", "sar_free_rows",
 ]
 
 
@@ -178,6 +178,8 @@ class Library:
             "sar_probe_streams": (c_int, [vp, c_int, P(ProbeJob), u64, c_int, P(ProbeResult)]),
             "sar_spread_yardstick": (c_int, [P(ctypes.c_float), ctypes.c_float, P(ctypes.c_float)]),
             "sar_spread_is_elsewhere": (c_int, [ctypes.c_float, ctypes.c_float]),
+            "sar_alloc_rows": (c_int, [vp, c_int, u64, P(vp), P(c_int), P(c_int)]),
+            "sar_free_rows": (c_int, [vp]),
         }
         assert sorted(sig) == sorted(EXPORTS)
         for name, (res, args) in sig.items():
@@ -370,6 +372,16 @@ class Context:
         p = ctypes.c_void_p()
         self._c(self._lib.lib.sar_rank_pointer(self._h, rank, ctypes.byref(p)))
         return int(p.value)
+
+    def alloc_rows(self, n: int, bytes_per_row: int):
+        """n rows back to back in one virtual range, owned by the context: (address of row 0, whether the two halves
+        of the rows lie in different regions of HBM, the SAR_SPREAD_* reason).  Adopt the row addresses to run on them."""
+        p, placed, reason = ctypes.c_void_p(), ctypes.c_int(0), ctypes.c_int(0)
+        self._c(self._lib.lib.sar_alloc_rows(self._h, n, bytes_per_row, ctypes.byref(p), ctypes.byref(placed), ctypes.byref(reason)))
+        return int(p.value), bool(placed.value), int(reason.value)
+
+    def free_rows(self):
+        self._c(self._lib.lib.sar_free_rows(self._h))
 
     @property
     def elems(self) -> int:

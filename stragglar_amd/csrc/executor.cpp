@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -94,6 +95,15 @@ struct sar_ctx {
     char* pair_lo = nullptr;           // the spread arena's two allocations, pair_bytes each, found to lie in
     char* pair_hi = nullptr;           // different regions of HBM; kept for the life of the context
     uint64_t pair_bytes = 0;
+    // sar_alloc_rows: n rows back to back in ONE virtual range.  Placed: two physical allocations of rows_half bytes
+    // each, found to lie in different regions of HBM, mapped next to each other at rows_va (the rows straddle the
+    // junction); kept for the life of the context.  Else a plain allocation.
+    char* rows_va = nullptr;
+    uint64_t rows_half = 0;
+    hipMemGenericAllocationHandle_t rows_lo_h{}, rows_hi_h{};
+    char* rows_plain = nullptr;
+    char* rows_base = nullptr;         // what the caller holds (null: none handed out)
+    uint64_t rows_bytes = 0;
     bool spread_capable = false;       // the device is one whose regions are known (MI355X, 288 GiB)
     int spread_reason = SAR_SPREAD_OFF;            // why the ranks sit where they sit (SAR_SPREAD_*)
     int spread_candidates = 0;                     // what the last search for a pair saw: allocations probed,
@@ -201,7 +211,14 @@ bool spread_is_elsewhere(float yardstick_ms, float probe_ms_value) { return prob
 // region's worth of candidates is held at a time beyond the pair.  Nothing is assumed about the order in which
 // the driver hands out memory, and a wrong verdict costs speed, not correctness: without a pair the caller falls
 // back to one allocation.  Returns a SAR_SPREAD_* reason.
-int find_spread_pair(sar_ctx* c, uint64_t bytes) {
+// Where the search gets its candidates: hipMalloc / hipFree for the rank arena, mapped physical allocations for
+// sar_alloc_rows.  `get` returns null when there is no more memory.
+struct CandidateSource {
+    std::function<char*(uint64_t)> get;
+    std::function<void(char*)> give_back;
+};
+
+int find_spread_pair(sar_ctx* c, uint64_t bytes, const CandidateSource& src, char** pair_lo, char** pair_hi) {
     const uint64_t window = 4 * kProbeStream;
     c->spread_candidates = 0; c->spread_same_ms = c->spread_pair_ms = 0.f; c->spread_search_bytes = 0;
     if (bytes < 8 * window) return SAR_SPREAD_NO_PAIR;
@@ -221,7 +238,7 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     float same = -1.f;
     uint64_t used = 0;
     for (int attempt = 0; attempt < 2 && used + bytes <= budget; ++attempt) {
-        if (hipMalloc((void**)&lo, bytes) != hipSuccess) { (void)hipGetLastError(); lo = nullptr; break; }
+        if (!(lo = src.get(bytes))) break;
         used += bytes;
         float adj[3];
         for (int k = 0; k < 3; ++k) adj[k] = probe_ms(c, lo + (uint64_t)(2 * k) * window, lo + (uint64_t)(2 * k + 1) * window, 3);
@@ -234,12 +251,12 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     }
     char* hi = nullptr;
     for (; lo && same > 0.f && used + bytes <= budget; used += bytes) {
-        char* cand = nullptr;
-        if (hipMalloc((void**)&cand, bytes) != hipSuccess) { (void)hipGetLastError(); break; }
+        char* cand = src.get(bytes);
+        if (!cand) break;
         c->spread_candidates += 1;
         const float t = probe_ms(c, lo, cand, 3);
         if (debug) std::fprintf(stderr, "sar spread: candidate %d %p %.1f us (limit %.1f us)\n", c->spread_candidates, (void*)cand, t * 1e3, kSpreadFaster * same * 1e3);
-        if (t < 0.f) { (void)hipFree(cand); break; }
+        if (t < 0.f) { src.give_back(cand); break; }
         if (spread_is_elsewhere(same, t)) {
             const float t2 = probe_ms(c, lo + bytes - window, cand + bytes - window, 3);
             if (debug) std::fprintf(stderr, "sar spread: candidate %d, other windows %.1f us\n", c->spread_candidates, t2 * 1e3);
@@ -249,10 +266,21 @@ int find_spread_pair(sar_ctx* c, uint64_t bytes) {
     }
     c->spread_same_ms = std::max(same, 0.f);
     c->spread_search_bytes = used;
-    for (char* p : held) (void)hipFree(p);
-    if (!hi) { if (lo) (void)hipFree(lo); return lo ? SAR_SPREAD_NO_PAIR : SAR_SPREAD_NO_MEMORY; }
-    c->pair_lo = lo; c->pair_hi = hi; c->pair_bytes = bytes;
+    for (char* p : held) src.give_back(p);
+    if (!hi) { if (lo) src.give_back(lo); return lo ? SAR_SPREAD_NO_PAIR : SAR_SPREAD_NO_MEMORY; }
+    *pair_lo = lo; *pair_hi = hi;
     return SAR_SPREAD_FOUND;
+}
+
+// The rank arena's pair: two hipMalloc allocations.
+int find_arena_pair(sar_ctx* c, uint64_t bytes) {
+    CandidateSource src;
+    src.get = [](uint64_t b) -> char* { char* p = nullptr; if (hipMalloc((void**)&p, b) != hipSuccess) { (void)hipGetLastError(); return nullptr; } return p; };
+    src.give_back = [](char* p) { (void)hipFree(p); };
+    char* lo = nullptr; char* hi = nullptr;
+    const int reason = find_spread_pair(c, bytes, src, &lo, &hi);
+    if (reason == SAR_SPREAD_FOUND) { c->pair_lo = lo; c->pair_hi = hi; c->pair_bytes = bytes; }
+    return reason;
 }
 
 void drop_ranks(sar_ctx* c) {
@@ -262,6 +290,97 @@ void drop_ranks(sar_ctx* c) {
     if (c->snapshot) { (void)hipFree(c->snapshot); c->snapshot = nullptr; }
     c->adopted.clear();
     c->n = 0; c->bytes_per_rank = 0; c->stride = 0;
+}
+
+// ---- rows in one virtual range (sar_alloc_rows) --------------------------------------------------------
+// A physical allocation mapped read-write at a virtual address of its own.
+struct VmBlock { char* va = nullptr; uint64_t bytes = 0; hipMemGenericAllocationHandle_t h{}; };
+
+hipMemAccessDesc vm_access(int device) {
+    hipMemAccessDesc acc{};
+    acc.location.type = hipMemLocationTypeDevice; acc.location.id = device; acc.flags = hipMemAccessFlagsProtReadWrite;
+    return acc;
+}
+
+// False when any step fails; nothing is left behind then.
+bool vm_block_create(int device, uint64_t bytes, VmBlock* out) {
+    hipMemAllocationProp prop{};
+    prop.type = hipMemAllocationTypePinned; prop.location.type = hipMemLocationTypeDevice; prop.location.id = device;
+    VmBlock b; b.bytes = bytes;
+    if (hipMemCreate(&b.h, bytes, &prop, 0) != hipSuccess) { (void)hipGetLastError(); return false; }
+    void* va = nullptr;
+    if (hipMemAddressReserve(&va, bytes, kArenaAlign, nullptr, 0) != hipSuccess || !va) { (void)hipGetLastError(); (void)hipMemRelease(b.h); return false; }
+    if (hipMemMap(va, bytes, 0, b.h, 0) != hipSuccess) { (void)hipGetLastError(); (void)hipMemAddressFree(va, bytes); (void)hipMemRelease(b.h); return false; }
+    const hipMemAccessDesc acc = vm_access(device);
+    if (hipMemSetAccess(va, bytes, &acc, 1) != hipSuccess) {
+        (void)hipGetLastError(); (void)hipMemUnmap(va, bytes); (void)hipMemAddressFree(va, bytes); (void)hipMemRelease(b.h); return false;
+    }
+    b.va = (char*)va; *out = b;
+    return true;
+}
+
+// Takes the block out of the address space; the physical allocation goes as well unless the caller keeps its handle.
+void vm_block_unmap(VmBlock& b, bool keep_handle) {
+    if (b.va) { (void)hipMemUnmap(b.va, b.bytes); (void)hipMemAddressFree(b.va, b.bytes); b.va = nullptr; }
+    if (!keep_handle) (void)hipMemRelease(b.h);
+}
+
+// Everything sar_alloc_rows holds.  Nothing on the device may still be using it.
+void release_rows(sar_ctx* c) {
+    if (c->rows_va) {
+        (void)hipMemUnmap(c->rows_va, 2 * c->rows_half);
+        (void)hipMemRelease(c->rows_lo_h); (void)hipMemRelease(c->rows_hi_h);
+        (void)hipMemAddressFree(c->rows_va, 2 * c->rows_half);
+    }
+    if (c->rows_plain) (void)hipFree(c->rows_plain);
+    c->rows_va = c->rows_plain = c->rows_base = nullptr; c->rows_half = c->rows_bytes = 0;
+}
+
+// Two physical allocations of `half` bytes each in different regions of HBM, mapped side by side at c->rows_va.
+// Returns a SAR_SPREAD_* reason; on anything but SAR_SPREAD_FOUND nothing is held.
+int map_rows_pair(sar_ctx* c, uint64_t half) {
+    std::vector<VmBlock> live;
+    live.reserve(64);
+    CandidateSource src;
+    src.get = [&](uint64_t b) -> char* {
+        VmBlock blk;
+        if (live.size() == live.capacity() || !vm_block_create(c->device, b, &blk)) return nullptr;
+        live.push_back(blk);
+        return blk.va;
+    };
+    src.give_back = [&](char* p) {
+        for (size_t i = 0; i < live.size(); ++i)
+            if (live[i].va == p) { vm_block_unmap(live[i], false); live.erase(live.begin() + (long)i); return; }
+    };
+    char* lo = nullptr; char* hi = nullptr;
+    const int reason = find_spread_pair(c, half, src, &lo, &hi);
+    if (reason != SAR_SPREAD_FOUND) { for (VmBlock& b : live) vm_block_unmap(b, false); return reason; }
+    VmBlock blo, bhi;
+    for (VmBlock& b : live) { if (b.va == lo) blo = b; else if (b.va == hi) bhi = b; else vm_block_unmap(b, false); }
+    // the probes have completed (probe_ms waits for each); the pair moves into one range, lo first
+    vm_block_unmap(blo, true); vm_block_unmap(bhi, true);
+    void* va = nullptr;
+    bool ok = hipMemAddressReserve(&va, 2 * half, kArenaAlign, nullptr, 0) == hipSuccess && va;
+    bool m0 = false, m1 = false;
+    if (ok) ok = m0 = hipMemMap(va, half, 0, blo.h, 0) == hipSuccess;
+    if (ok) ok = m1 = hipMemMap((char*)va + half, half, 0, bhi.h, 0) == hipSuccess;
+    if (ok) { const hipMemAccessDesc acc = vm_access(c->device); ok = hipMemSetAccess(va, 2 * half, &acc, 1) == hipSuccess; }
+    if (!ok) {
+        (void)hipGetLastError();
+        if (m0) (void)hipMemUnmap(va, half);
+        if (m1) (void)hipMemUnmap((char*)va + half, half);
+        if (va) (void)hipMemAddressFree(va, 2 * half);
+        (void)hipMemRelease(blo.h); (void)hipMemRelease(bhi.h);
+        return SAR_SPREAD_NO_MEMORY;
+    }
+    c->rows_va = (char*)va; c->rows_half = half; c->rows_lo_h = blo.h; c->rows_hi_h = bhi.h;
+    return SAR_SPREAD_FOUND;
+}
+
+bool rows_adopted(const sar_ctx* c) {
+    if (!c->rows_base) return false;
+    for (const char* p : c->adopted) if (p >= c->rows_base && p < c->rows_base + c->rows_bytes) return true;
+    return false;
 }
 
 // A byte interval of one rank buffer that a row reads or writes.
@@ -822,6 +941,7 @@ void sar_destroy(sar_ctx* c) {
     if (c->prework_stream) (void)hipStreamSynchronize(c->prework_stream);
     drop_ranks(c);
     drop_pair(c);
+    release_rows(c);
     for (auto e : c->ev_prof) (void)hipEventDestroy(e);
     if (c->d_flag) (void)hipFree(c->d_flag);
     if (c->ev_start) (void)hipEventDestroy(c->ev_start);
@@ -852,7 +972,7 @@ static int alloc_ranks_body(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtyp
     if (reason == SAR_SPREAD_FOUND) {
         uint64_t need = kSpreadMinAlloc;
         while (need < stride * (uint64_t)half) need <<= 1;
-        if (c->pair_bytes < need) { drop_pair(c); reason = need <= kSpreadMaxAlloc ? find_spread_pair(c, need) : SAR_SPREAD_TOO_LARGE; }
+        if (c->pair_bytes < need) { drop_pair(c); reason = need <= kSpreadMaxAlloc ? find_arena_pair(c, need) : SAR_SPREAD_TOO_LARGE; }
     }
     const bool spread = reason == SAR_SPREAD_FOUND;
     c->spread_reason = reason;
@@ -912,6 +1032,15 @@ static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_
     if (!c) return set_error(SAR_EINVAL, "context is null");
     SAR_HIP(hipSetDevice(c->device));
     int rc = check_rank_pointers(c->device, n, device_ptrs, bytes_per_rank, dtype); if (rc) return rc;
+    // the context's own arena is given back below: pointers into it would be left dangling
+    if (c->arena) {
+        const uint64_t lo_span = c->arena_hi ? c->pair_bytes : c->stride * (uint64_t)c->n;
+        for (int r = 0; r < n; ++r) {
+            const char* p = (const char*)device_ptrs[r];
+            if ((p >= c->arena && p < c->arena + lo_span) || (c->arena_hi && p >= c->arena_hi && p < c->arena_hi + c->pair_bytes))
+                return set_error(SAR_EINVAL, "a rank pointer lies in this context's own rank arena, which adoption gives back");
+        }
+    }
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_ranks(c);
     for (int r = 0; r < n; ++r) c->adopted.push_back((char*)device_ptrs[r]);
@@ -922,6 +1051,58 @@ static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_
 
 int sar_adopt_ranks(sar_ctx* c, int n, void* const* device_ptrs, uint64_t bytes_per_rank, int dtype) {
     return guarded([&] { return adopt_ranks_body(c, n, device_ptrs, bytes_per_rank, dtype); });
+}
+
+// n rows of bytes_per_row bytes back to back in one virtual range; see sar.h.
+static int alloc_rows_body(sar_ctx* c, int n, uint64_t bytes_per_row, void** base, int* placed, int* reason_out) {
+    if (!c || !base) return set_error(SAR_EINVAL, "null argument");
+    *base = nullptr;
+    if (placed) *placed = 0;
+    if (n < 2 || n > SAR_MAX_RANKS) return set_error(SAR_EINVAL, "n out of range");
+    if (bytes_per_row == 0 || bytes_per_row > SAR_MAX_RANK_BYTES) return set_error(SAR_EINVAL, "bytes_per_row out of range");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    SAR_HIP(hipStreamSynchronize(c->prework_stream));
+    if (rows_adopted(c)) drop_ranks(c);                       // the rows those rank buffers were go away
+    if (c->rows_plain) { (void)hipFree(c->rows_plain); c->rows_plain = nullptr; }
+    c->rows_base = nullptr; c->rows_bytes = 0;
+    const uint64_t total = (uint64_t)n * bytes_per_row, lo_bytes = (uint64_t)((n + 1) / 2) * bytes_per_row;
+    int reason = !c->tune.arena_spread ? SAR_SPREAD_OFF : !c->spread_capable ? SAR_SPREAD_UNKNOWN_DEVICE :
+                 total < kSpreadMinPayload ? SAR_SPREAD_SMALL_PAYLOAD : SAR_SPREAD_FOUND;
+    if (reason == SAR_SPREAD_FOUND) {
+        uint64_t need = kSpreadMinAlloc;
+        while (need < lo_bytes) need <<= 1;
+        if (need > kSpreadMaxAlloc) reason = SAR_SPREAD_TOO_LARGE;
+        else if (c->rows_half < need) { release_rows(c); reason = map_rows_pair(c, need); }
+    }
+    if (reason == SAR_SPREAD_FOUND) {
+        c->rows_base = c->rows_va + c->rows_half - lo_bytes;      // rows [0, ceil(n/2)) end where the second allocation begins
+    } else {
+        hipError_t e = hipMalloc((void**)&c->rows_plain, total);
+        if (e != hipSuccess && c->rows_va) { (void)hipGetLastError(); release_rows(c); e = hipMalloc((void**)&c->rows_plain, total); }
+        if (e != hipSuccess) { (void)hipGetLastError(); c->rows_plain = nullptr; return set_error(SAR_ENOMEM, std::string("rows: ") + hipGetErrorString(e)); }
+        c->rows_base = c->rows_plain;
+    }
+    c->rows_bytes = total;
+    *base = c->rows_base;
+    if (placed) *placed = reason == SAR_SPREAD_FOUND ? 1 : 0;
+    if (reason_out) *reason_out = reason;
+    return SAR_OK;
+}
+
+int sar_alloc_rows(sar_ctx* c, int n, uint64_t bytes_per_row, void** base, int* placed, int* reason) {
+    return guarded([&] { return alloc_rows_body(c, n, bytes_per_row, base, placed, reason); });
+}
+
+int sar_free_rows(sar_ctx* c) {
+    if (!c) return set_error(SAR_EINVAL, "context is null");
+    SAR_HIP(hipSetDevice(c->device));
+    SAR_HIP(hipStreamSynchronize(c->stream));
+    SAR_HIP(hipStreamSynchronize(c->prework_stream));
+    if (rows_adopted(c)) drop_ranks(c);
+    if (c->rows_plain) { (void)hipFree(c->rows_plain); c->rows_plain = nullptr; }
+    c->rows_base = nullptr; c->rows_bytes = 0;               // a placed pair stays mapped for the next sar_alloc_rows
+    return SAR_OK;
 }
 
 static int check_rank_range(sar_ctx* c, int rank, uint64_t off, uint64_t bytes) {

@@ -85,6 +85,7 @@ class EmulatedGroup:
             raise ValueError("invalid schedule: " + reason)
         self._key = None
         self._placed = None            # ((numel, dtype), tensors) of the last rank_tensors call while its memory is in use
+        self.block_placed = False      # whether the last rank_block lies in two regions of HBM
 
     def close(self):
         self._ctx.close()
@@ -119,6 +120,27 @@ class EmulatedGroup:
         self._key = (tuple(ptrs), numel * es, name)
         self._placed = ((numel, name), tuple(out))
         return out
+
+    def rank_block(self, numel: int, dtype):
+        """ONE tensor ``[world_size, numel]`` whose rows are the emulated ranks' flat buffers (row r = rank r), in memory
+        the library allocates (``sar_alloc_rows``): one virtual range, so it is an ordinary contiguous tensor, whose two
+        halves are physical allocations in different regions of HBM from 128 MiB in all -- the placement that
+        ``rank_tensors`` gives separate tensors, for callers that keep the ranks as the rows of one tensor (what
+        ``dist.all_reduce`` takes through ``stragglar_amd.c10d_backend``).  Valid until the next ``rank_block`` call or
+        ``close``."""
+        import torch
+        name = _TORCH_DTYPES.get(str(dtype))
+        if name is None:
+            raise TypeError("unsupported dtype %s" % dtype)
+        es = capi.ELEM_SIZE[name]
+        if self._placed is None:
+            self._key = None                           # rank buffers adopted from the previous block go with it
+        base, placed, _reason = self._ctx.alloc_rows(self.n, numel * es)
+        typestr = {"f32": "<f4", "f16": "<f2", "bf16": "<i2"}[name]
+        t = torch.as_tensor(_DeviceArray(base, self.n * numel, typestr), device="cuda:%d" % self.device)
+        t = (t.view(torch.bfloat16) if name == "bf16" else t).view(self.n, numel)
+        self.block_placed = placed
+        return t
 
     def _order(self, tensors):
         """Rank order seen by the schedule: the straggler takes the last place."""

@@ -570,6 +570,37 @@ def test_adopted_buffers_must_be_long_enough(gpu_ctx, sarlib):
         other.close()
 
 
+def test_rows_in_one_virtual_range(gpu_ctx, sarlib, oracle):
+    """sar_alloc_rows: n rows back to back at one address range that belongs to the context, adopted as rank buffers;
+    results as on any other buffers; the rows and what was adopted from them go together."""
+    import stragglar_amd as sa
+    n, dtype = 8, "f32"
+    ctx = gpu_ctx
+    for elems in (7 * 8 * 75000 + 5, 7 * 100):              # 134 MB in all (placed on a 288 GiB device); a few KB
+        inputs = make_inputs(n, elems, dtype, seed=elems % 97)
+        want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+        base, placed, reason = ctx.alloc_rows(n, elems * 4)
+        assert base and (reason == 3 or placed == (n * elems * 4 >= 128 << 20)), reason
+        ctx.adopt_ranks([base + r * elems * 4 for r in range(n)], elems * 4, dtype)
+        assert [ctx.rank_pointer(r) for r in range(n)] == [base + r * elems * 4 for r in range(n)]
+        for executor in (1, 0):
+            ctx.set_tuning(**dict(ctx.default_tuning, executor=executor))
+            for r, x in enumerate(inputs):
+                ctx.upload(r, x)
+            ctx.prepare(sarlib.parse(read_golden("stragglar_n8_cu.txt"), n), sarlib.builtin("prework_rs", n))
+            ctx.run(0.0)
+            for r in range(n):
+                assert_bits_equal(ctx.download(r), want[r], "%d elements executor %d rank %d" % (elems, executor, r))
+    ctx.free_rows()
+    with pytest.raises(sa.SarError) as ei:                  # the adopted rank buffers went with the rows
+        ctx.run(-1.0)
+    assert ei.value.code == -7
+    with pytest.raises(sa.SarError):
+        ctx.alloc_rows(1, 4096)
+    with pytest.raises(sa.SarError):
+        ctx.alloc_rows(n, 0)
+
+
 def gather_slices(ctx, rank, chunk, parts, offs, length):
     """The same `length` elements at each offset of every chunk of one rank, downloaded piecewise."""
     es = ES[ctx.dtype]

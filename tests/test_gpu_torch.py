@@ -279,3 +279,61 @@ def test_data_parallel_step_through_dist_all_reduce(c10d_group):
         got = torch.cat([p.grad.reshape(-1) for p in replicas[r].parameters()]).double()
         assert torch.allclose(got, want, rtol=1e-6, atol=1e-9), "replica %d" % r
         assert torch.equal(flat[r], flat[0])                           # every replica holds the same bits
+
+
+def test_rank_block_is_one_tensor_in_two_regions(oracle):
+    """EmulatedGroup.rank_block: the emulated ranks as the rows of ONE contiguous tensor in memory the library maps
+    (sar_alloc_rows: two physical allocations in different regions of HBM side by side in one virtual range), worked
+    on in place, bit for bit the checker's result; a small block is a plain allocation."""
+    from stragglar_amd.capi import SPREAD_REASONS
+    from stragglar_amd.torch_emulation import EmulatedGroup
+    n = 8
+    group = EmulatedGroup(n, straggler_rank=6)
+    try:
+        for numel, dtype, name in ((7 * 8 * 160000, torch.float32, "f32"), (7 * 512, torch.float32, "f32"), (7 * 8 * 160000, torch.bfloat16, "bf16")):
+            y = group.rank_block(numel, dtype)
+            assert y.shape == (n, numel) and y.dtype == dtype and y.is_cuda and y.is_contiguous()
+            assert y[1].data_ptr() - y[0].data_ptr() == numel * dtype.itemsize
+            _, placed, reason = group._ctx.alloc_rows(n, numel * dtype.itemsize)        # the same request again: same verdict
+            y = group.rank_block(numel, dtype)
+            big = n * numel * dtype.itemsize >= 128 << 20
+            if reason != 3:                                  # 3: not a 288 GiB device, regions unknown
+                assert placed == big and group.block_placed == big, SPREAD_REASONS.get(reason, "?")
+            g = torch.Generator(device="cpu").manual_seed(11)
+            y.copy_((torch.rand(n, numel, generator=g, dtype=torch.float32) * 2 - 1).to(dtype))
+            inputs = [to_np_bits(y[r]).copy() for r in range(n)]
+            group.all_reduce([y[r] for r in range(n)])
+            group.all_reduce([y[r] for r in range(n)])        # the second call finds the rows adopted and sums the sums
+            order = list(range(n))
+            order[6], order[7] = order[7], order[6]
+            want = [inputs[i].copy() for i in order]
+            for _ in range(2):
+                oracle.run("stragglar", want, name, rounds=parse_table(read_golden("synth_pow2_n8.txt")), delay=0.0)
+            for k, i in enumerate(order):
+                assert_bits_equal(to_np_bits(y[i]), want[k], "%s %d rank %d" % (name, numel, i))
+        # tensors of the library's own arena, in another order than they were handed out, are refused rather than
+        # adopted (adoption gives the arena back)
+        import stragglar_amd as sa
+        ts = group.rank_tensors(7 * 1024, torch.float32)
+        with pytest.raises(sa.SarError, match="own rank arena"):
+            group.all_reduce(ts[::-1])
+    finally:
+        group.close()
+
+
+def test_dist_all_reduce_on_rows_the_library_placed(c10d_group):
+    """empty_ranks: the [n, numel] tensor for dist.all_reduce in memory of the library's (two regions of HBM from
+    128 MiB in all); the result as for any other tensor."""
+    import torch.distributed as dist
+    n = 8
+    numel = c10d_group.padded_numel(5_000_000, n, 4)                  # 160 MB in all
+    y = c10d_group.empty_ranks(n, numel)
+    assert y.shape == (n, numel) and y.is_contiguous()
+    y.copy_((torch.arange(n * numel, device="cuda") % 13).reshape(n, numel).float())
+    want = y.sum(dim=0, keepdim=True).expand(n, numel).clone()        # small integers: exact in any order
+    dist.all_reduce(y)
+    assert torch.equal(y, want)
+    z = c10d_group.empty_ranks(4, 3 * 256, torch.float16)             # another rank count has a block of its own
+    z.fill_(1.0)
+    dist.all_reduce(z)
+    assert torch.all(z == 4.0) and torch.equal(y, want)
