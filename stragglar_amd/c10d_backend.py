@@ -16,6 +16,7 @@ ONE process (world size 1 as far as torch is concerned) and carries all emulated
     sb.configure(straggler_rank=6)                       # STRAGGLER_RANK of dummy.cpp:157, dp.py:22
     dist.init_process_group("stragglar", store=dist.HashStore(), rank=0, world_size=1)
     y = torch.empty(8, sb.padded_numel(numel, 8, 4), device="cuda")      # row r = emulated rank r's buffer
+    y = sb.empty_ranks(8, sb.padded_numel(numel, 8, 4))                  # or: the same tensor in memory the library placed
     dist.all_reduce(y)                                   # every row now holds the sum over the rows
 
 ``all_reduce`` takes one 2-D tensor ``[n, numel]`` whose n rows are the n emulated ranks' flat buffers and works
