@@ -36,8 +36,9 @@ constexpr uint64_t kSpreadMinPayload = 128ull << 20;   // spread arena: from 16 
 constexpr uint64_t kSpreadHeadroom = 16ull << 30;      // memory left alone while looking for the pair
 constexpr uint64_t kSpreadMinAlloc = 8ull << 30, kSpreadMaxAlloc = 32ull << 30;      // per half; one size serves most payloads
 constexpr uint64_t kSpreadSearch = 96ull << 30;        // candidates held while looking, beyond the pair itself: one region
-constexpr float kSpreadFaster = 0.94f;                 // a pair in different regions takes at most this fraction of the fastest pair within one
-                                                       // (measured 0.87 to 0.895; candidates in the same region 1.0 and more)
+constexpr float kSpreadFaster = 0.95f;                 // a pair in different regions takes at most this fraction of the fastest pair within one
+                                                       // (measured 0.85 to 0.895 on an empty device, up to 0.932 with other allocations around;
+                                                       // candidates in the same region 0.98 and more)
 constexpr float kSpreadStraddle = 0.86f;               // the two ends of an allocation against its neighbouring windows: below this a boundary runs through it
                                                        // (measured 0.80 with a boundary, 0.90 to 0.93 without)
 constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 streams of this size (beyond what the Infinity Cache absorbs)

@@ -811,6 +811,15 @@ def test_spread_arena(gpu_ctx, sarlib, oracle):
     elems = 7 * 8 * 75000 + 5                       # 16.8 MB per rank: 134 MB of payload
     inputs = make_inputs(n, elems, dtype, seed=77)
     want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
+    # a context of its own: the search and its figures are this test's, not left over from larger rank buffers of a
+    # test before (the shared context keeps the pair it found for those)
+    gpu_ctx.alloc_ranks(2, 4096, "f32")
+    with sarlib.context(0) as own:
+        own.default_tuning = gpu_ctx.default_tuning
+        spread_arena_checks(own, sarlib, n, dtype, elems, inputs, want)
+
+
+def spread_arena_checks(gpu_ctx, sarlib, n, dtype, elems, inputs, want):
     seen = []
     for spread in (1, 0, 1):
         for executor in (1, 0):
@@ -837,7 +846,7 @@ def test_spread_arena(gpu_ctx, sarlib, oracle):
     print(why)
     if st.spread_reason != 3:                    # 3: not a 288 GiB device, regions unknown
         assert seen[0] == 1 and st.spread_reason == 0, why
-        assert 0 < st.spread_pair_ms < 0.94 * st.spread_same_ms, why          # the search's own limit; measured 0.87 to 0.895, a pair in one region 1.0 and more
+        assert 0 < st.spread_pair_ms < 0.95 * st.spread_same_ms, why          # the search's own limit; measured 0.85 to 0.932, a pair in one region 0.98 and more
         assert st.spread_search_bytes <= (96 + 2 * 8 + 1) << 30, why
     # small payloads stay back to back
     small = make_inputs(n, 7 * 8 * 100, dtype, seed=78)
