@@ -573,9 +573,14 @@ def test_adopted_buffers_must_be_long_enough(gpu_ctx, sarlib):
 def test_rows_in_one_virtual_range(gpu_ctx, sarlib, oracle):
     """sar_alloc_rows: n rows back to back at one address range that belongs to the context, adopted as rank buffers;
     results as on any other buffers; the rows and what was adopted from them go together."""
+    with sarlib.context(0) as own:                          # its own: the pair it maps goes when it closes
+        own.default_tuning = gpu_ctx.default_tuning
+        rows_checks(own, sarlib, oracle)
+
+
+def rows_checks(ctx, sarlib, oracle):
     import stragglar_amd as sa
     n, dtype = 8, "f32"
-    ctx = gpu_ctx
     for elems in (7 * 8 * 75000 + 5, 7 * 100):              # 134 MB in all (placed on a 288 GiB device); a few KB
         inputs = make_inputs(n, elems, dtype, seed=elems % 97)
         want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
@@ -670,10 +675,12 @@ def test_rank_buffers_beyond_4gib(gpu_ctx, sarlib, oracle, executor):
     ring's eight and the upper fifth of direct's whole-buffer rows lie beyond 4 GiB."""
     nbytes = sarlib.pad_bytes(5 << 30, 8)
     assert nbytes > 1 << 32
-    try:
-        full_size_all_algorithms(gpu_ctx, sarlib, oracle, executor, nbytes, seed=7000)
-    finally:
-        gpu_ctx.alloc_ranks(2, 4096, "f32")      # give the 80 GiB back before the next test
+    # in a context of its own, which takes its 80 GiB and the 2 x 32 GiB of its spread arena along when it closes
+    # (the shared context would keep that pair, and the search figures that go with it, for the tests that follow)
+    gpu_ctx.alloc_ranks(2, 4096, "f32")
+    with sarlib.context(0) as own:
+        own.default_tuning = gpu_ctx.default_tuning
+        full_size_all_algorithms(own, sarlib, oracle, executor, nbytes, seed=7000)
 
 
 def test_config3_bf16_1gib_with_delay(gpu_ctx, sarlib, oracle):
@@ -811,15 +818,6 @@ def test_spread_arena(gpu_ctx, sarlib, oracle):
     elems = 7 * 8 * 75000 + 5                       # 16.8 MB per rank: 134 MB of payload
     inputs = make_inputs(n, elems, dtype, seed=77)
     want = run_oracle(oracle, "stragglar", inputs, dtype, read_golden("stragglar_n8_cu.txt"), delay=0.0)
-    # a context of its own: the search and its figures are this test's, not left over from larger rank buffers of a
-    # test before (the shared context keeps the pair it found for those)
-    gpu_ctx.alloc_ranks(2, 4096, "f32")
-    with sarlib.context(0) as own:
-        own.default_tuning = gpu_ctx.default_tuning
-        spread_arena_checks(own, sarlib, n, dtype, elems, inputs, want)
-
-
-def spread_arena_checks(gpu_ctx, sarlib, n, dtype, elems, inputs, want):
     seen = []
     for spread in (1, 0, 1):
         for executor in (1, 0):
