@@ -297,8 +297,9 @@ def test_rank_block_is_one_tensor_in_two_regions(oracle):
             _, placed, reason = group._ctx.alloc_rows(n, numel * dtype.itemsize)        # the same request again: same verdict
             y = group.rank_block(numel, dtype)
             big = n * numel * dtype.itemsize >= 128 << 20
-            if reason != 3:                                  # 3: not a 288 GiB device, regions unknown
-                assert placed == big and group.block_placed == big, SPREAD_REASONS.get(reason, "?")
+            # (that a block of this size IS placed on a 288 GiB device is asserted where the entry point is tested by
+            # itself, tests/test_gpu_parity.py::test_rows_in_one_virtual_range; here other contexts hold memory around it)
+            assert placed == (reason == 0) and group.block_placed == placed and (big or not placed), SPREAD_REASONS.get(reason, "?")
             g = torch.Generator(device="cpu").manual_seed(11)
             y.copy_((torch.rand(n, numel, generator=g, dtype=torch.float32) * 2 - 1).to(dtype))
             inputs = [to_np_bits(y[r]).copy() for r in range(n)]
