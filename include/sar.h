@@ -56,9 +56,10 @@ enum {
     SAR_SPREAD_SMALL_PAYLOAD = 2,  /* less than 128 MiB over all ranks: the caches carry the schedule */
     SAR_SPREAD_UNKNOWN_DEVICE = 3, /* not a 288 GiB MI355X: the regions of this device are not known */
     SAR_SPREAD_NO_MEMORY = 4,      /* too little free device memory to look for a pair */
-    SAR_SPREAD_NO_PAIR = 5,        /* no candidate was clearly faster against the first allocation than that is against itself */
+    SAR_SPREAD_NO_PAIR = 5,        /* the probe times of the candidates did not fall into two populations with a clear gap */
     SAR_SPREAD_TOO_LARGE = 6,      /* half the ranks take more than 32 GiB */
-    SAR_SPREAD_ADOPTED = 7         /* caller-owned buffers (sar_adopt_ranks) are taken where they are */
+    SAR_SPREAD_ADOPTED = 7,        /* caller-owned buffers (sar_adopt_ranks) are taken where they are */
+    SAR_SPREAD_POOL_BUSY = 8       /* the GPU's pair of allocations has no room left beside the leases other contexts hold */
 };
 
 #define SAR_MAX_RANKS 64
@@ -105,6 +106,11 @@ typedef struct sar_stats_t {
     uint64_t spread_search_bytes;  /* the most device memory held at a time while looking, the pair included      */
     uint64_t fused_forwarded_bytes;    /* the same two figures for the single launch of pre-work + main schedule  */
     uint64_t fused_elided_store_bytes; /* (fused_prework = 1), out of algorithmic_bytes + prework_bytes           */
+    uint64_t placed_pool_bytes;    /* the GPU's pair of allocations in different regions of HBM, shared by all     */
+    int32_t placed_pool_contexts;  /* contexts of the process: its size (both together) and the contexts attached  */
+    int32_t main_launches;         /* `launches` split: kernel launches of the main schedule ...                  */
+    int32_t prework_launches;      /* ... and of the pre-work when it runs on its own (beside a delay, or in front */
+                                   /* of the schedule when there is no single launch for both)                    */
 } sar_stats_t;
 
 /* run-time tunables of the executors; sar_get_tuning() reports the defaults */
@@ -394,6 +400,11 @@ int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64
  * (clearly below the yardstick), else 0.  Negative = SAR_EINVAL. */
 int sar_spread_yardstick(const float* neighbours_ms, float ends_ms, float* yardstick_ms);
 int sar_spread_is_elsewhere(float yardstick_ms, float probe_ms);
+/* The verdict on a whole search: probe_ms[0..n) are the candidates' times against the first allocation.  Returns 1 and
+ * *pick = the candidate to take when the times fall into two populations with a clear gap -- candidates elsewhere,
+ * clearly below the yardstick, and the rest at the yardstick and above, nothing in between --, else 0 and *pick = -1:
+ * the ranks then sit in one ordinary allocation (SAR_SPREAD_NO_PAIR).  Times <= 0 are failed probes and say nothing. */
+int sar_spread_pick(float yardstick_ms, const float* probe_ms, int n, int* pick);
 
 /* Ticks of the device's constant-rate wall clock that delay_ms lasts: the
  * figure the CLI prints as "Sleep cycles" (calculate_sleep_cycles,

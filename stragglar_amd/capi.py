@@ -19,7 +19,7 @@ _LIB_PATH = os.path.join(_HERE, "lib", "libsar_hip.so")
 DTYPES = {"f32": 0, "f16": 1, "bf16": 2}
 ELEM_SIZE = {"f32": 4, "f16": 2, "bf16": 2}
 OP_KINDS = {0: "copy", 1: "xreduce", 2: "reduce_into", 3: "mreduce"}
-SPREAD_REASONS = {0: "found", 1: "off", 2: "small payload", 3: "unknown device", 4: "no memory", 5: "no pair", 6: "too large", 7: "adopted"}
+SPREAD_REASONS = {0: "found", 1: "off", 2: "small payload", 3: "unknown device", 4: "no memory", 5: "no pair", 6: "too large", 7: "adopted", 8: "pool busy"}
 
 
 class SarError(RuntimeError):
@@ -45,7 +45,9 @@ class Stats(ctypes.Structure):
                 ("forwarded_bytes", ctypes.c_uint64), ("fused_prework", ctypes.c_int32), ("arena_spread", ctypes.c_int32),
                 ("elided_store_bytes", ctypes.c_uint64), ("spread_reason", ctypes.c_int32), ("spread_candidates", ctypes.c_int32),
                 ("spread_same_ms", ctypes.c_float), ("spread_pair_ms", ctypes.c_float), ("spread_search_bytes", ctypes.c_uint64),
-                ("fused_forwarded_bytes", ctypes.c_uint64), ("fused_elided_store_bytes", ctypes.c_uint64)]
+                ("fused_forwarded_bytes", ctypes.c_uint64), ("fused_elided_store_bytes", ctypes.c_uint64),
+                ("placed_pool_bytes", ctypes.c_uint64), ("placed_pool_contexts", ctypes.c_int32),
+                ("main_launches", ctypes.c_int32), ("prework_launches", ctypes.c_int32)]
 
 
 class PlanRow(ctypes.Structure):
@@ -117,7 +119,7 @@ EXPORTS = [
     "sar_ranks_identical", "sar_get_tuning", "sar_set_tuning", "sar_prepare", "sar_run", "sar_run_profiled",
     "sar_launch_bytes", "sar_sleep_ticks", "sar_stats", "sar_plan", "sar_plan_rows", "sar_default_tuning",
     "sar_run_static", "sar_static_scratch_bytes", "sar_rank_pointer", "sar_probe_streams",
-    "sar_spread_yardstick", "sar_spread_is_elsewhere", "sar_alloc_rows", "sar_free_rows",
+    "sar_spread_yardstick", "sar_spread_is_elsewhere", "sar_spread_pick", "sar_alloc_rows", "sar_free_rows",
 ]
 
 
@@ -178,6 +180,7 @@ class Library:
             "sar_probe_streams": (c_int, [vp, c_int, P(ProbeJob), u64, c_int, P(ProbeResult)]),
             "sar_spread_yardstick": (c_int, [P(ctypes.c_float), ctypes.c_float, P(ctypes.c_float)]),
             "sar_spread_is_elsewhere": (c_int, [ctypes.c_float, ctypes.c_float]),
+            "sar_spread_pick": (c_int, [ctypes.c_float, P(ctypes.c_float), c_int, P(c_int)]),
             "sar_alloc_rows": (c_int, [vp, c_int, u64, P(vp), P(c_int), P(c_int)]),
             "sar_free_rows": (c_int, [vp]),
         }
@@ -214,6 +217,16 @@ class Library:
         if rc < 0:
             self.check(rc)
         return bool(rc)
+
+    def spread_pick(self, yardstick_ms: float, probe_ms) -> int:
+        """The candidate a search would take given all candidates' probe times (ms), or -1 when the times do not fall
+        into two populations with a clear gap."""
+        arr = (ctypes.c_float * max(1, len(probe_ms)))(*probe_ms)
+        pick = ctypes.c_int(-1)
+        rc = self.lib.sar_spread_pick(yardstick_ms, arr, len(probe_ms), ctypes.byref(pick))
+        if rc < 0:
+            self.check(rc)
+        return pick.value
 
     def default_tuning(self) -> "Tuning":
         t = Tuning()

@@ -224,7 +224,7 @@ int main(int argc, char* argv[]) {
         double mean = sum_ms / numIters;
         fprintf(stderr, "# bytes_to_memory=%.0f mean_ms=%.4f min_ms=%.4f memory_GBps=%.1f (best %.1f) frac_of_8TBps=%.3f algorithmic_bytes=%.0f algorithmic_GBps=%.1f launches=%d graph=%d\n",
                 to_memory, mean, min_ms, to_memory / mean / 1e6, to_memory / min_ms / 1e6, to_memory / mean / 1e6 / 8000.0, algorithmic, algorithmic / mean / 1e6,
-                one_launch ? 1 : st.launches - ((st.prework_bytes > 0 && !with_prework) ? 1 : 0), st.uses_graph);
+                one_launch ? 1 : st.main_launches + (with_prework ? st.prework_launches : 0), st.uses_graph);
         fprintf(stderr, "# executor=%s components=%d column_threads=%d value_slots=%d taken_from_LDS_bytes=%.0f stores_left_out_bytes=%.0f prework=%s ranks_in_two_hbm_regions=%d\n",
                 st.executor ? "column" : "rounds", st.col_components, st.col_block, st.col_slots,
                 one_launch ? (double)st.fused_forwarded_bytes : (double)st.forwarded_bytes, one_launch ? (double)st.fused_elided_store_bytes : (double)st.elided_store_bytes,

@@ -15,6 +15,7 @@
 
 #include "column_plan.hpp"
 #include "kernels.hpp"
+#include "placed_pool.hpp"
 #include "sar.h"
 #include "schedule.hpp"
 
@@ -33,15 +34,6 @@ int set_error(int code, const std::string& msg) { g_error = msg; return code; }
 
 constexpr uint64_t kArenaAlign = 2ull << 20;   // rank bases on 2 MiB boundaries (one large-page fragment each)
 constexpr uint64_t kSpreadMinPayload = 128ull << 20;   // spread arena: from 16 MiB per rank at n = 8 (below, the caches carry the schedule)
-constexpr uint64_t kSpreadHeadroom = 16ull << 30;      // memory left alone while looking for the pair
-constexpr uint64_t kSpreadMinAlloc = 8ull << 30, kSpreadMaxAlloc = 32ull << 30;      // per half; one size serves most payloads
-constexpr uint64_t kSpreadSearch = 96ull << 30;        // candidates held while looking, beyond the pair itself: one region
-constexpr float kSpreadFaster = 0.95f;                 // a pair in different regions takes at most this fraction of the fastest pair within one
-                                                       // (measured 0.85 to 0.895 on an empty device, up to 0.932 with other allocations around;
-                                                       // candidates in the same region 0.98 and more)
-constexpr float kSpreadStraddle = 0.86f;               // the two ends of an allocation against its neighbouring windows: below this a boundary runs through it
-                                                       // (measured 0.80 with a boundary, 0.90 to 0.93 without)
-constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 streams of this size (beyond what the Infinity Cache absorbs)
 constexpr float kMaxDelayMs = 60000.f;
 
 // One kernel launch: the rows of a round that share a kernel (COPY /
@@ -93,23 +85,16 @@ struct sar_ctx {
     char* arena = nullptr;             // ranks [0, split) at arena + r * stride
     char* arena_hi = nullptr;          // ranks [split, n) at arena_hi + (r - split) * stride (spread arena only)
     int split = 0;
-    char* pair_lo = nullptr;           // the spread arena's two allocations, pair_bytes each, found to lie in
-    char* pair_hi = nullptr;           // different regions of HBM; kept for the life of the context
-    uint64_t pair_bytes = 0;
-    // sar_alloc_rows: n rows back to back in ONE virtual range.  Placed: two physical allocations of rows_half bytes
-    // each, found to lie in different regions of HBM, mapped next to each other at rows_va (the rows straddle the
-    // junction); kept for the life of the context.  Else a plain allocation.
-    char* rows_va = nullptr;
-    uint64_t rows_half = 0;
-    hipMemGenericAllocationHandle_t rows_lo_h{}, rows_hi_h{};
+    // Placed memory comes from the GPU's pair of allocations in different regions of HBM (placed_pool.hpp), which all
+    // contexts of the process share: an arena lease (ranks [0, split) in the lower allocation, the rest in the upper
+    // one) and a lease for sar_alloc_rows (n rows back to back across the junction of the two).  Otherwise `arena` and
+    // `rows_plain` are ordinary allocations of this context.
+    bool pool_attached = false, arena_leased = false, rows_leased = false;
     char* rows_plain = nullptr;
     char* rows_base = nullptr;         // what the caller holds (null: none handed out)
     uint64_t rows_bytes = 0;
     bool spread_capable = false;       // the device is one whose regions are known (MI355X, 288 GiB)
     int spread_reason = SAR_SPREAD_OFF;            // why the ranks sit where they sit (SAR_SPREAD_*)
-    int spread_candidates = 0;                     // what the last search for a pair saw: allocations probed,
-    float spread_same_ms = 0.f, spread_pair_ms = 0.f;      // the probe's time within one region and for the pair kept,
-    uint64_t spread_search_bytes = 0;              // most memory held at a time
     char* snapshot = nullptr;
     int* d_flag = nullptr;
 
@@ -162,220 +147,35 @@ void drop_plan(sar_ctx* c) {
     c->stats = sar_stats_t{};
 }
 
-void drop_pair(sar_ctx* c) {
-    if (c->pair_lo) (void)hipFree(c->pair_lo);
-    if (c->pair_hi) (void)hipFree(c->pair_hi);
-    c->pair_lo = c->pair_hi = nullptr; c->pair_bytes = 0;
+sar::ProbeEnv probe_env(const sar_ctx* c) { return sar::ProbeEnv{c->device, c->stream, c->wall_khz}; }
+
+void attach_pool(sar_ctx* c) {
+    if (!c->pool_attached) { sar::pool_attach(c->device, c); c->pool_attached = true; }
 }
 
-// Best of `reps` runs of the region probe on two windows of 4 * kProbeStream bytes, in milliseconds as the kernel
-// timed itself on the device's wall clock; negative on error.
-float probe_ms(sar_ctx* c, char* a, char* b, int reps) {
-    unsigned long long* stamps = nullptr;
-    if (hipMalloc((void**)&stamps, 2 * sizeof(unsigned long long)) != hipSuccess) { (void)hipGetLastError(); return -1.f; }
-    float best = -1.f;
-    for (int i = 0; i < reps; ++i) {
-        unsigned long long h[2] = {~0ull, 0ull};
-        if (hipMemcpyAsync(stamps, h, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-            sar::launch_region_probe(c->stream, a, b, kProbeStream, stamps) != hipSuccess ||
-            hipMemcpyAsync(h, stamps, sizeof(h), hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-            hipStreamSynchronize(c->stream) != hipSuccess || h[1] <= h[0]) { (void)hipGetLastError(); best = -1.f; break; }
-        const float ms = (float)((double)(h[1] - h[0]) / (double)c->wall_khz);
-        if (best < 0.f || ms < best) best = ms;
-    }
-    (void)hipFree(stamps);
-    return best;
-}
-
-// The two decisions of the region search as functions of probe times alone, so that they can be checked against
-// recorded times without a device (sar_spread_yardstick, sar_spread_is_elsewhere).
-// Yardstick: the fastest of the four pairs of windows within the first allocation.  Returns false when the
-// allocation's two ends probe like different regions against its median neighbouring pair: a boundary runs through it.
-bool spread_yardstick(const float neighbours_ms[3], float ends_ms, float* yardstick_ms) {
-    float adj[3] = {neighbours_ms[0], neighbours_ms[1], neighbours_ms[2]};
-    std::sort(adj, adj + 3);
-    *yardstick_ms = std::min(ends_ms, adj[0]);
-    return !(ends_ms < kSpreadStraddle * adj[1]);
-}
-bool spread_is_elsewhere(float yardstick_ms, float probe_ms_value) { return probe_ms_value > 0.f && probe_ms_value < kSpreadFaster * yardstick_ms; }
-
-// Two allocations of `bytes` each that lie in different regions of HBM.  Measured on MI355X: the 288 GiB behave as
-// three regions of 96 GiB (presumably the stack levels of the 12-high HBM3E), and streams that run at the same
-// time in different regions get in each other's way less: the write-heavy schedules here gain 15 to 25 %, and
-// which region a buffer falls in is all that matters, not where in it.  Where an allocation lands physically is
-// the driver's business, so candidates are allocated one after the other and each is timed against the first
-// with a short probe (eight write streams of 128 MiB, four in either allocation) until one turns out to lie
-// elsewhere; the others are given back.  The yardstick is the probe's own time for windows that do share a
-// region, not a fixed figure: the fastest of four pairs of windows of the first allocation (three neighbouring
-// pairs and its two ends; measured 181-213 us, candidates in the same region 183-217 us, elsewhere 158-162 us).
-// Elsewhere means at most kSpreadFaster of that fastest pair, twice, on different windows of both.  At most one
-// region's worth of candidates is held at a time beyond the pair.  Nothing is assumed about the order in which
-// the driver hands out memory, and a wrong verdict costs speed, not correctness: without a pair the caller falls
-// back to one allocation.  Returns a SAR_SPREAD_* reason.
-// Where the search gets its candidates: hipMalloc / hipFree for the rank arena, mapped physical allocations for
-// sar_alloc_rows.  `get` returns null when there is no more memory.
-struct CandidateSource {
-    std::function<char*(uint64_t)> get;
-    std::function<void(char*)> give_back;
-};
-
-int find_spread_pair(sar_ctx* c, uint64_t bytes, const CandidateSource& src, char** pair_lo, char** pair_hi) {
-    const uint64_t window = 4 * kProbeStream;
-    c->spread_candidates = 0; c->spread_same_ms = c->spread_pair_ms = 0.f; c->spread_search_bytes = 0;
-    if (bytes < 8 * window) return SAR_SPREAD_NO_PAIR;
-    size_t free_b = 0, total_b = 0;
-    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); return SAR_SPREAD_NO_MEMORY; }
-    if (free_b < 4 * bytes + kSpreadHeadroom) return SAR_SPREAD_NO_MEMORY;
-    // enough candidates to cross a region boundary from anywhere, no more
-    const uint64_t budget = std::min<uint64_t>((uint64_t)free_b - kSpreadHeadroom, kSpreadSearch + 2 * bytes);
-    std::vector<char*> held;
-    try { held.reserve((size_t)(budget / bytes) + 2); } catch (const std::bad_alloc&) { return SAR_SPREAD_NO_MEMORY; }      // no allocation below
-    const bool debug = std::getenv("SAR_DEBUG_SPREAD") != nullptr;
-    // The first allocation and the yardstick.  Should a region boundary run through the allocation, its two ends
-    // probe like a pair in different regions while its neighbouring windows do not (ends at most kSpreadStraddle of
-    // the median neighbouring pair; without a boundary the ends take 0.90 to 0.93 of it): the allocation then stays
-    // held as a spacer and the one behind it takes its place.
-    char* lo = nullptr;
-    float same = -1.f;
-    uint64_t used = 0;
-    for (int attempt = 0; attempt < 2 && used + bytes <= budget; ++attempt) {
-        if (!(lo = src.get(bytes))) break;
-        used += bytes;
-        float adj[3];
-        for (int k = 0; k < 3; ++k) adj[k] = probe_ms(c, lo + (uint64_t)(2 * k) * window, lo + (uint64_t)(2 * k + 1) * window, 3);
-        const float ends = probe_ms(c, lo, lo + bytes - window, 3);
-        if (adj[0] <= 0.f || adj[1] <= 0.f || adj[2] <= 0.f || ends <= 0.f) { same = -1.f; break; }
-        if (debug) std::fprintf(stderr, "sar spread: first allocation %p, neighbouring windows %.1f %.1f %.1f us, ends %.1f us\n", (void*)lo, adj[0] * 1e3, adj[1] * 1e3, adj[2] * 1e3, ends * 1e3);
-        const bool whole = spread_yardstick(adj, ends, &same);
-        if (!whole && attempt == 0) { held.push_back(lo); lo = nullptr; same = -1.f; continue; }
-        break;
-    }
-    char* hi = nullptr;
-    for (; lo && same > 0.f && used + bytes <= budget; used += bytes) {
-        char* cand = src.get(bytes);
-        if (!cand) break;
-        c->spread_candidates += 1;
-        const float t = probe_ms(c, lo, cand, 3);
-        if (debug) std::fprintf(stderr, "sar spread: candidate %d %p %.1f us (limit %.1f us)\n", c->spread_candidates, (void*)cand, t * 1e3, kSpreadFaster * same * 1e3);
-        if (t < 0.f) { src.give_back(cand); break; }
-        if (spread_is_elsewhere(same, t)) {
-            const float t2 = probe_ms(c, lo + bytes - window, cand + bytes - window, 3);
-            if (debug) std::fprintf(stderr, "sar spread: candidate %d, other windows %.1f us\n", c->spread_candidates, t2 * 1e3);
-            if (spread_is_elsewhere(same, t2)) { hi = cand; c->spread_pair_ms = std::max(t, t2); used += bytes; break; }
-        }
-        held.push_back(cand);
-    }
-    c->spread_same_ms = std::max(same, 0.f);
-    c->spread_search_bytes = used;
-    for (char* p : held) src.give_back(p);
-    if (!hi) { if (lo) src.give_back(lo); return lo ? SAR_SPREAD_NO_PAIR : SAR_SPREAD_NO_MEMORY; }
-    *pair_lo = lo; *pair_hi = hi;
-    return SAR_SPREAD_FOUND;
-}
-
-// The rank arena's pair: two hipMalloc allocations.
-int find_arena_pair(sar_ctx* c, uint64_t bytes) {
-    CandidateSource src;
-    src.get = [](uint64_t b) -> char* { char* p = nullptr; if (hipMalloc((void**)&p, b) != hipSuccess) { (void)hipGetLastError(); return nullptr; } return p; };
-    src.give_back = [](char* p) { (void)hipFree(p); };
-    char* lo = nullptr; char* hi = nullptr;
-    const int reason = find_spread_pair(c, bytes, src, &lo, &hi);
-    if (reason == SAR_SPREAD_FOUND) { c->pair_lo = lo; c->pair_hi = hi; c->pair_bytes = bytes; }
-    return reason;
-}
-
+// The rank buffers go.  A lease goes back to the pool only once the whole device is idle: a caller's own kernels on
+// streams of its own may still be working on addresses it got from sar_rank_pointer.
 void drop_ranks(sar_ctx* c) {
     drop_plan(c);
-    if (c->arena && c->arena != c->pair_lo) (void)hipFree(c->arena);
-    c->arena = c->arena_hi = nullptr; c->split = 0;
+    if (c->arena && c->arena_leased) { (void)hipDeviceSynchronize(); sar::pool_release_arena(c->device, c); }
+    else if (c->arena) (void)hipFree(c->arena);
+    c->arena = c->arena_hi = nullptr; c->split = 0; c->arena_leased = false;
     if (c->snapshot) { (void)hipFree(c->snapshot); c->snapshot = nullptr; }
     c->adopted.clear();
     c->n = 0; c->bytes_per_rank = 0; c->stride = 0;
 }
 
 // ---- rows in one virtual range (sar_alloc_rows) --------------------------------------------------------
-// A physical allocation mapped read-write at a virtual address of its own.
-struct VmBlock { char* va = nullptr; uint64_t bytes = 0; hipMemGenericAllocationHandle_t h{}; };
-
-hipMemAccessDesc vm_access(int device) {
-    hipMemAccessDesc acc{};
-    acc.location.type = hipMemLocationTypeDevice; acc.location.id = device; acc.flags = hipMemAccessFlagsProtReadWrite;
-    return acc;
-}
-
-// False when any step fails; nothing is left behind then.
-bool vm_block_create(int device, uint64_t bytes, VmBlock* out) {
-    hipMemAllocationProp prop{};
-    prop.type = hipMemAllocationTypePinned; prop.location.type = hipMemLocationTypeDevice; prop.location.id = device;
-    VmBlock b; b.bytes = bytes;
-    if (hipMemCreate(&b.h, bytes, &prop, 0) != hipSuccess) { (void)hipGetLastError(); return false; }
-    void* va = nullptr;
-    if (hipMemAddressReserve(&va, bytes, kArenaAlign, nullptr, 0) != hipSuccess || !va) { (void)hipGetLastError(); (void)hipMemRelease(b.h); return false; }
-    if (hipMemMap(va, bytes, 0, b.h, 0) != hipSuccess) { (void)hipGetLastError(); (void)hipMemAddressFree(va, bytes); (void)hipMemRelease(b.h); return false; }
-    const hipMemAccessDesc acc = vm_access(device);
-    if (hipMemSetAccess(va, bytes, &acc, 1) != hipSuccess) {
-        (void)hipGetLastError(); (void)hipMemUnmap(va, bytes); (void)hipMemAddressFree(va, bytes); (void)hipMemRelease(b.h); return false;
-    }
-    b.va = (char*)va; *out = b;
-    return true;
-}
-
-// Takes the block out of the address space; the physical allocation goes as well unless the caller keeps its handle.
-void vm_block_unmap(VmBlock& b, bool keep_handle) {
-    if (b.va) { (void)hipMemUnmap(b.va, b.bytes); (void)hipMemAddressFree(b.va, b.bytes); b.va = nullptr; }
-    if (!keep_handle) (void)hipMemRelease(b.h);
-}
-
-// Everything sar_alloc_rows holds.  Nothing on the device may still be using it.
+// Everything sar_alloc_rows holds.  The whole device is drained first: a caller's kernels on streams of its own (a
+// torch tensor over these rows) may still be touching the memory.
 void release_rows(sar_ctx* c) {
-    if (c->rows_va) {
-        (void)hipMemUnmap(c->rows_va, 2 * c->rows_half);
-        (void)hipMemRelease(c->rows_lo_h); (void)hipMemRelease(c->rows_hi_h);
-        (void)hipMemAddressFree(c->rows_va, 2 * c->rows_half);
+    if (c->rows_leased || c->rows_plain) (void)hipDeviceSynchronize();
+    if (c->rows_leased) sar::pool_release_rows(c->device, c);
+    if (c->rows_plain) {
+        const hipError_t e = hipFree(c->rows_plain);
+        if (e != hipSuccess) { (void)hipGetLastError(); if (std::getenv("SAR_DEBUG")) std::fprintf(stderr, "sar: releasing rows: hipFree: %s\n", hipGetErrorString(e)); }
     }
-    if (c->rows_plain) (void)hipFree(c->rows_plain);
-    c->rows_va = c->rows_plain = c->rows_base = nullptr; c->rows_half = c->rows_bytes = 0;
-}
-
-// Two physical allocations of `half` bytes each in different regions of HBM, mapped side by side at c->rows_va.
-// Returns a SAR_SPREAD_* reason; on anything but SAR_SPREAD_FOUND nothing is held.
-int map_rows_pair(sar_ctx* c, uint64_t half) {
-    std::vector<VmBlock> live;
-    live.reserve(64);
-    CandidateSource src;
-    src.get = [&](uint64_t b) -> char* {
-        VmBlock blk;
-        if (live.size() == live.capacity() || !vm_block_create(c->device, b, &blk)) return nullptr;
-        live.push_back(blk);
-        return blk.va;
-    };
-    src.give_back = [&](char* p) {
-        for (size_t i = 0; i < live.size(); ++i)
-            if (live[i].va == p) { vm_block_unmap(live[i], false); live.erase(live.begin() + (long)i); return; }
-    };
-    char* lo = nullptr; char* hi = nullptr;
-    const int reason = find_spread_pair(c, half, src, &lo, &hi);
-    if (reason != SAR_SPREAD_FOUND) { for (VmBlock& b : live) vm_block_unmap(b, false); return reason; }
-    VmBlock blo, bhi;
-    for (VmBlock& b : live) { if (b.va == lo) blo = b; else if (b.va == hi) bhi = b; else vm_block_unmap(b, false); }
-    // the probes have completed (probe_ms waits for each); the pair moves into one range, lo first
-    vm_block_unmap(blo, true); vm_block_unmap(bhi, true);
-    void* va = nullptr;
-    bool ok = hipMemAddressReserve(&va, 2 * half, kArenaAlign, nullptr, 0) == hipSuccess && va;
-    bool m0 = false, m1 = false;
-    if (ok) ok = m0 = hipMemMap(va, half, 0, blo.h, 0) == hipSuccess;
-    if (ok) ok = m1 = hipMemMap((char*)va + half, half, 0, bhi.h, 0) == hipSuccess;
-    if (ok) { const hipMemAccessDesc acc = vm_access(c->device); ok = hipMemSetAccess(va, 2 * half, &acc, 1) == hipSuccess; }
-    if (!ok) {
-        (void)hipGetLastError();
-        if (m0) (void)hipMemUnmap(va, half);
-        if (m1) (void)hipMemUnmap((char*)va + half, half);
-        if (va) (void)hipMemAddressFree(va, 2 * half);
-        (void)hipMemRelease(blo.h); (void)hipMemRelease(bhi.h);
-        return SAR_SPREAD_NO_MEMORY;
-    }
-    c->rows_va = (char*)va; c->rows_half = half; c->rows_lo_h = blo.h; c->rows_hi_h = bhi.h;
-    return SAR_SPREAD_FOUND;
+    c->rows_plain = c->rows_base = nullptr; c->rows_bytes = 0; c->rows_leased = false;
 }
 
 bool rows_adopted(const sar_ctx* c) {
@@ -755,10 +555,11 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     if (prework) sar::byte_counts(prework->s, c->elems(), elem_size_of(c->dtype), &st.prework_bytes, nullptr);
     st.rounds = (int)main_sched->s.rounds.size();
     for (const auto& r : main_sched->s.rounds) st.ops += (int)r.size();
-    if (column) st.launches += 1;
-    else for (const auto& L : c->rounds) st.launches += L.total_tiles ? 1 : 0;
-    if (pre_column) st.launches += 1;
-    else for (const auto& L : c->prework) st.launches += L.total_tiles ? 1 : 0;
+    if (column) st.main_launches = 1;
+    else for (const auto& L : c->rounds) st.main_launches += L.total_tiles ? 1 : 0;
+    if (pre_column) st.prework_launches = 1;
+    else for (const auto& L : c->prework) st.prework_launches += L.total_tiles ? 1 : 0;
+    st.launches = st.main_launches + st.prework_launches;
     st.executor = column ? 1 : 0;
     st.col_block = column ? (int32_t)cp.block : 0;
     st.col_slots = column ? (int32_t)cp.nslots : 0;
@@ -768,8 +569,12 @@ sar_stats_t plan_stats(const sar_ctx* c, const sar_schedule* prework, const sar_
     st.fused_prework = fused ? 1 : 0;
     if (fused && fp) { st.fused_forwarded_bytes = fp->forwarded_bytes; st.fused_elided_store_bytes = fp->elided_bytes; }
     st.arena_spread = c->spread() ? 1 : 0;
-    st.spread_reason = c->spread_reason; st.spread_candidates = c->spread_candidates;
-    st.spread_same_ms = c->spread_same_ms; st.spread_pair_ms = c->spread_pair_ms; st.spread_search_bytes = c->spread_search_bytes;
+    st.spread_reason = c->spread_reason;
+    if (c->pool_attached) {
+        const sar::SearchRecord rec = sar::pool_record(c->device);
+        st.spread_candidates = rec.candidates; st.spread_same_ms = rec.same_ms; st.spread_pair_ms = rec.pair_ms;
+        st.spread_search_bytes = rec.search_bytes; st.placed_pool_bytes = rec.pool_bytes; st.placed_pool_contexts = rec.users;
+    }
     return st;
 }
 
@@ -941,8 +746,8 @@ void sar_destroy(sar_ctx* c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     if (c->prework_stream) (void)hipStreamSynchronize(c->prework_stream);
     drop_ranks(c);
-    drop_pair(c);
     release_rows(c);
+    if (c->pool_attached) sar::pool_detach(c->device, c);        // the last context to go takes the pair along
     for (auto e : c->ev_prof) (void)hipEventDestroy(e);
     if (c->d_flag) (void)hipFree(c->d_flag);
     if (c->ev_start) (void)hipEventDestroy(c->ev_start);
@@ -963,30 +768,28 @@ static int alloc_ranks_body(sar_ctx* c, int n, uint64_t bytes_per_rank, int dtyp
     SAR_HIP(hipStreamSynchronize(c->stream));
     drop_ranks(c);
     uint64_t stride = (bytes_per_rank + kArenaAlign - 1) / kArenaAlign * kArenaAlign;
-    // Spread arena: half the ranks in an allocation of their own that lies in another region of HBM than the
-    // first half's (find_spread_pair).  Only for payloads that are bound by memory, and only when the device has
-    // the room to look for such a pair; otherwise the ranks sit back to back.
+    // Spread arena: half the ranks in the other of the GPU's two allocations that were found to lie in different
+    // regions of HBM (placed_pool.hpp).  Only for payloads that are bound by memory, and only when the device has the
+    // room to look for such a pair; otherwise the ranks sit back to back in an allocation of this context's own.
     const int half = (n + 1) / 2;
     const uint64_t payload = stride * (uint64_t)n;
     int reason = !c->tune.arena_spread ? SAR_SPREAD_OFF : !c->spread_capable ? SAR_SPREAD_UNKNOWN_DEVICE :
                  payload < kSpreadMinPayload ? SAR_SPREAD_SMALL_PAYLOAD : SAR_SPREAD_FOUND;
     if (reason == SAR_SPREAD_FOUND) {
-        uint64_t need = kSpreadMinAlloc;
-        while (need < stride * (uint64_t)half) need <<= 1;
-        if (c->pair_bytes < need) { drop_pair(c); reason = need <= kSpreadMaxAlloc ? find_arena_pair(c, need) : SAR_SPREAD_TOO_LARGE; }
+        attach_pool(c);
+        reason = sar::pool_lease_arena(probe_env(c), c, stride * (uint64_t)half, stride * (uint64_t)(n - half), &c->arena, &c->arena_hi);
     }
-    const bool spread = reason == SAR_SPREAD_FOUND;
     c->spread_reason = reason;
-    if (spread) {
-        c->arena = c->pair_lo; c->arena_hi = c->pair_hi; c->split = half;
+    if (reason == SAR_SPREAD_FOUND) {
+        c->split = half; c->arena_leased = true;
     } else {
         hipError_t e = hipMalloc((void**)&c->arena, payload);
-        if (e != hipSuccess && c->pair_lo) {       // the idle spread arena may be what is in the way
-            (void)hipGetLastError(); drop_pair(c);
+        if (e != hipSuccess && sar::pool_trim(c->device)) {       // the idle pair may be what is in the way
+            (void)hipGetLastError();
             e = hipMalloc((void**)&c->arena, payload);
         }
         if (e != hipSuccess) { (void)hipGetLastError(); c->arena = nullptr; return set_error(SAR_ENOMEM, std::string("rank arena: ") + hipGetErrorString(e)); }
-        c->arena_hi = nullptr; c->split = n;
+        c->arena_hi = nullptr; c->split = n; c->arena_leased = false;
     }
     c->n = n; c->dtype = dtype; c->bytes_per_rank = bytes_per_rank; c->stride = stride;
     return SAR_OK;
@@ -1035,10 +838,10 @@ static int adopt_ranks_body(sar_ctx* c, int n, void* const* device_ptrs, uint64_
     int rc = check_rank_pointers(c->device, n, device_ptrs, bytes_per_rank, dtype); if (rc) return rc;
     // the context's own arena is given back below: pointers into it would be left dangling
     if (c->arena) {
-        const uint64_t lo_span = c->arena_hi ? c->pair_bytes : c->stride * (uint64_t)c->n;
+        const uint64_t lo_span = c->stride * (uint64_t)(c->arena_leased ? c->split : c->n), hi_span = c->stride * (uint64_t)(c->n - c->split);
         for (int r = 0; r < n; ++r) {
             const char* p = (const char*)device_ptrs[r];
-            if ((p >= c->arena && p < c->arena + lo_span) || (c->arena_hi && p >= c->arena_hi && p < c->arena_hi + c->pair_bytes))
+            if ((p >= c->arena && p < c->arena + lo_span) || (c->arena_hi && p >= c->arena_hi && p < c->arena_hi + hi_span))
                 return set_error(SAR_EINVAL, "a rank pointer lies in this context's own rank arena, which adoption gives back");
         }
     }
@@ -1065,22 +868,20 @@ static int alloc_rows_body(sar_ctx* c, int n, uint64_t bytes_per_row, void** bas
     SAR_HIP(hipStreamSynchronize(c->stream));
     SAR_HIP(hipStreamSynchronize(c->prework_stream));
     if (rows_adopted(c)) drop_ranks(c);                       // the rows those rank buffers were go away
-    if (c->rows_plain) { (void)hipFree(c->rows_plain); c->rows_plain = nullptr; }
-    c->rows_base = nullptr; c->rows_bytes = 0;
+    release_rows(c);
     const uint64_t total = (uint64_t)n * bytes_per_row, lo_bytes = (uint64_t)((n + 1) / 2) * bytes_per_row;
     int reason = !c->tune.arena_spread ? SAR_SPREAD_OFF : !c->spread_capable ? SAR_SPREAD_UNKNOWN_DEVICE :
                  total < kSpreadMinPayload ? SAR_SPREAD_SMALL_PAYLOAD : SAR_SPREAD_FOUND;
     if (reason == SAR_SPREAD_FOUND) {
-        uint64_t need = kSpreadMinAlloc;
-        while (need < lo_bytes) need <<= 1;
-        if (need > kSpreadMaxAlloc) reason = SAR_SPREAD_TOO_LARGE;
-        else if (c->rows_half < need) { release_rows(c); reason = map_rows_pair(c, need); }
+        // rows [0, ceil(n/2)) end where the second allocation begins
+        attach_pool(c);
+        reason = sar::pool_lease_rows(probe_env(c), c, lo_bytes, total - lo_bytes, &c->rows_base);
     }
     if (reason == SAR_SPREAD_FOUND) {
-        c->rows_base = c->rows_va + c->rows_half - lo_bytes;      // rows [0, ceil(n/2)) end where the second allocation begins
+        c->rows_leased = true;
     } else {
         hipError_t e = hipMalloc((void**)&c->rows_plain, total);
-        if (e != hipSuccess && c->rows_va) { (void)hipGetLastError(); release_rows(c); e = hipMalloc((void**)&c->rows_plain, total); }
+        if (e != hipSuccess && sar::pool_trim(c->device)) { (void)hipGetLastError(); e = hipMalloc((void**)&c->rows_plain, total); }
         if (e != hipSuccess) { (void)hipGetLastError(); c->rows_plain = nullptr; return set_error(SAR_ENOMEM, std::string("rows: ") + hipGetErrorString(e)); }
         c->rows_base = c->rows_plain;
     }
@@ -1101,8 +902,7 @@ int sar_free_rows(sar_ctx* c) {
     SAR_HIP(hipStreamSynchronize(c->stream));
     SAR_HIP(hipStreamSynchronize(c->prework_stream));
     if (rows_adopted(c)) drop_ranks(c);
-    if (c->rows_plain) { (void)hipFree(c->rows_plain); c->rows_plain = nullptr; }
-    c->rows_base = nullptr; c->rows_bytes = 0;               // a placed pair stays mapped for the next sar_alloc_rows
+    release_rows(c);                                          // (the GPU's pair itself stays for the next call)
     return SAR_OK;
 }
 
@@ -1453,12 +1253,18 @@ static int probe_streams_body(sar_ctx* c, int njobs, const sar_probe_job* jobs, 
 int sar_spread_yardstick(const float* neighbours_ms, float ends_ms, float* yardstick_ms) {
     if (!neighbours_ms || !yardstick_ms) return set_error(SAR_EINVAL, "null argument");
     if (!(neighbours_ms[0] > 0.f && neighbours_ms[1] > 0.f && neighbours_ms[2] > 0.f && ends_ms > 0.f)) return set_error(SAR_EINVAL, "probe times must be positive");
-    return spread_yardstick(neighbours_ms, ends_ms, yardstick_ms) ? 0 : 1;
+    return sar::spread_yardstick(neighbours_ms, ends_ms, yardstick_ms) ? 0 : 1;
 }
 
 int sar_spread_is_elsewhere(float yardstick_ms, float probe_ms_value) {
     if (!(yardstick_ms > 0.f)) return set_error(SAR_EINVAL, "the yardstick must be positive");
-    return spread_is_elsewhere(yardstick_ms, probe_ms_value) ? 1 : 0;
+    return sar::spread_is_elsewhere(yardstick_ms, probe_ms_value) ? 1 : 0;
+}
+
+int sar_spread_pick(float yardstick_ms, const float* probe_ms, int n, int* pick) {
+    if (!(yardstick_ms > 0.f) || !probe_ms || n < 0 || !pick) return set_error(SAR_EINVAL, "bad argument");
+    *pick = n ? sar::spread_pick(yardstick_ms, probe_ms, n) : -1;
+    return *pick >= 0 ? 1 : 0;
 }
 
 int sar_probe_streams(sar_ctx* c, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out) {
@@ -1560,6 +1366,7 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 char* g_scratch_ptr[kMaxDevices] = {};      // device address of `scratch` on every GPU it was resolved on
+std::mutex g_static_run_mutex[kMaxDevices]; // one sar_run_static at a time per GPU: they all write the one array
 
 // The address of this GPU's copy of `scratch`, resolved once per device with that device current.
 int static_scratch(int device, char** out) {
@@ -1636,7 +1443,10 @@ int run_static_body(int device, void* stream, const sar_schedule* prework, const
     c.d_ops = (sar::DevOp*)base; c.d_ptrs = (char**)(base + ptrs_at);
     for (Launch& L : per_round) L.first_op -= (uint32_t)lo;
     // Copies and launches on the caller's stream.  Whatever happens, the stream is drained before the host copies of
-    // the tables go out of scope; the result is complete when it has.
+    // the tables go out of scope; the result is complete when it has.  Every call on this GPU writes the same array
+    // and its kernels read it until the stream has drained, so the calls take turns: the lock is held from the first
+    // copy until the drain (a second thread's call waits here; nothing is lost, the call blocks on its stream anyway).
+    std::lock_guard<std::mutex> turn(g_static_run_mutex[device]);
     auto enqueue = [&]() -> int {
         SAR_HIP(hipMemcpyAsync(base, rows.data() + lo, rows_b, hipMemcpyHostToDevice, st));
         if (ptrs_b) SAR_HIP(hipMemcpyAsync(base + ptrs_at, ptrs.data(), ptrs_b, hipMemcpyHostToDevice, st));

@@ -41,9 +41,12 @@ def padded_numel(numel: int, world_size: int, elem_size: int, parts: Optional[in
 
 
 class _DeviceArray:
-    """Device memory owned by the library, described for ``torch.as_tensor`` (no copy)."""
+    """Device memory owned by the library, described for ``torch.as_tensor`` (no copy).  torch keeps this object
+    alive for as long as the tensor's storage lives, and the object keeps the owning context: the memory is not
+    given back by garbage collection of the group while a tensor over it is still around."""
 
-    def __init__(self, ptr: int, numel: int, typestr: str):
+    def __init__(self, ptr: int, numel: int, typestr: str, owner):
+        self.owner = owner
         self.__cuda_array_interface__ = {"shape": (numel,), "typestr": typestr, "data": (ptr, False), "version": 2}
 
 
@@ -85,9 +88,24 @@ class EmulatedGroup:
             raise ValueError("invalid schedule: " + reason)
         self._key = None
         self._placed = None            # ((numel, dtype), tensors) of the last rank_tensors call while its memory is in use
+        self._block = None             # the tensor of the last rank_block call while its memory is in use
         self.block_placed = False      # whether the last rank_block lies in two regions of HBM
 
+    def _retire(self, tensors):
+        """Memory behind tensors that were handed out is about to go: wait for everything the device still does with it
+        (the caller's kernels run on torch's streams, which the library's own synchronisation does not cover), then
+        empty the tensors, so that a later touch is a Python error and not an access to freed device memory.  (Views
+        that the caller made of them keep the old address: they must not be used any more.)"""
+        import torch
+        torch.cuda.synchronize(self.device)
+        for t in tensors:
+            t.set_()
+
     def close(self):
+        if self._placed is not None:
+            self._retire(self._placed[1]); self._placed = None
+        if self._block is not None:
+            self._retire([self._block]); self._block = None
         self._ctx.close()
 
     def rank_tensors(self, numel: int, dtype) -> List:
@@ -95,8 +113,9 @@ class EmulatedGroup:
         itself (``sar_alloc_ranks``: from 128 MiB over all ranks, half the ranks in another region of HBM than the
         rest, which is worth 15 to 25 % of the bandwidth and which tensors that torch allocated next to each other
         cannot have).  The tensors alias the group's memory: they are valid until a ``rank_tensors`` call for another
-        size or dtype, an ``all_reduce`` on tensors of the caller's own, or ``close``; a call for the same size and
-        dtype returns the same tensors.  ``all_reduce`` on them skips the adoption step."""
+        size or dtype, an ``all_reduce`` on tensors of the caller's own, or ``close``, each of which waits for the device
+        and then leaves them empty; a call for the same size and dtype returns the same tensors.  ``all_reduce`` on them
+        skips the adoption step."""
         import torch
         name = _TORCH_DTYPES.get(str(dtype))
         if name is None:
@@ -104,7 +123,8 @@ class EmulatedGroup:
         es = capi.ELEM_SIZE[name]
         if self._placed is not None and self._placed[0] == (numel, name):
             return list(self._placed[1])               # the same buffers again: nothing to allocate or lower
-        self._placed = None
+        if self._placed is not None:
+            self._retire(self._placed[1]); self._placed = None
         self._ctx.alloc_ranks(self.n, numel * es, name)
         order = list(range(self.n))
         order[self.straggler], order[self.n - 1] = order[self.n - 1], order[self.straggler]
@@ -114,7 +134,7 @@ class EmulatedGroup:
         for k, i in enumerate(order):                   # schedule rank k is the caller's rank order[k]
             ptr = self._ctx.rank_pointer(k)
             ptrs.append(ptr)
-            t = torch.as_tensor(_DeviceArray(ptr, numel, typestr), device="cuda:%d" % self.device)
+            t = torch.as_tensor(_DeviceArray(ptr, numel, typestr, self._ctx), device="cuda:%d" % self.device)
             out[i] = t.view(torch.bfloat16) if name == "bf16" else t
         self._ctx.prepare(self._main, self._prework)
         self._key = (tuple(ptrs), numel * es, name)
@@ -127,7 +147,7 @@ class EmulatedGroup:
         halves are physical allocations in different regions of HBM from 128 MiB in all -- the placement that
         ``rank_tensors`` gives separate tensors, for callers that keep the ranks as the rows of one tensor (what
         ``dist.all_reduce`` takes through ``stragglar_amd.c10d_backend``).  Valid until the next ``rank_block`` call or
-        ``close``."""
+        ``close``, which wait for the device and leave the old tensor empty."""
         import torch
         name = _TORCH_DTYPES.get(str(dtype))
         if name is None:
@@ -135,11 +155,14 @@ class EmulatedGroup:
         es = capi.ELEM_SIZE[name]
         if self._placed is None:
             self._key = None                           # rank buffers adopted from the previous block go with it
+        if self._block is not None:
+            self._retire([self._block]); self._block = None
         base, placed, _reason = self._ctx.alloc_rows(self.n, numel * es)
         typestr = {"f32": "<f4", "f16": "<f2", "bf16": "<i2"}[name]
-        t = torch.as_tensor(_DeviceArray(base, self.n * numel, typestr), device="cuda:%d" % self.device)
+        t = torch.as_tensor(_DeviceArray(base, self.n * numel, typestr, self._ctx), device="cuda:%d" % self.device)
         t = (t.view(torch.bfloat16) if name == "bf16" else t).view(self.n, numel)
         self.block_placed = placed
+        self._block = t
         return t
 
     def _order(self, tensors):
@@ -172,7 +195,8 @@ class EmulatedGroup:
         nbytes = t0.numel() * t0.element_size()
         key = (tuple(t.data_ptr() for t in ordered), nbytes, dtype)
         if key != self._key:                       # new buffers: adopt them and lower the schedule onto them
-            self._placed = None                    # (the library's own rank memory goes when other buffers are adopted)
+            if self._placed is not None:           # (the library's own rank memory goes when other buffers are adopted)
+                self._retire(self._placed[1]); self._placed = None
             self._ctx.adopt_ranks(list(key[0]), nbytes, dtype)
             self._ctx.prepare(self._main, self._prework)
             self._key = key

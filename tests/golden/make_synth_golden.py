@@ -72,7 +72,7 @@ def main():
     except AssertionError as e:
         print("pow2 n=4 raises AssertionError as read from the source:", e)
     npow2 = load(ref, "synthesizer_nonpow2")
-    for n in (6, 10, 12, 14, 24):
+    for n in (6, 10, 12, 14, 24, 48):
         npow2.n = n
         gpus = [npow2.GPU(i, n) for i in range(n)]
         sched = npow2.construct_schedule(gpus)

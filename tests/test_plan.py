@@ -143,6 +143,7 @@ def test_prework_and_misaligned_buffers(sarlib):
     S = sarlib.pad_bytes(16 * MIB, 8)
     st = plan(sarlib, "stragglar", 8, S, delay=True)
     assert st.prework_bytes == 8 * S and st.launches == 2     # the pre-work as one launch, then the column kernel
+    assert (st.main_launches, st.prework_launches) == (1, 1)
     assert st.fused_prework == 1                              # ... or both as one launch when nobody is late
     assert plan(sarlib, "stragglar", 8, S, delay=True, col_fuse_prework=0).fused_prework == 0
     assert plan(sarlib, "stragglar", 8, S, delay=True, executor=0).fused_prework == 0
@@ -534,6 +535,27 @@ def test_region_search_decisions_on_recorded_probe_times(sarlib):
     assert straddles
     # ... and with such a yardstick nothing would pass, so the search sets the allocation aside instead of using it
     assert not sarlib.spread_is_elsewhere(y, 0.159)
+    # The verdict on a whole search: the candidates' times must fall into two populations with a clear gap.
+    for neighbours, ends, same_region, elsewhere in _RECORDED_SEARCHES:
+        y, _ = sarlib.spread_yardstick([t * 1e-3 for t in neighbours], ends * 1e-3)
+        times = [t * 1e-3 for t in same_region] + [elsewhere[0] * 1e-3]
+        assert sarlib.spread_pick(y, times) == len(times) - 1, (neighbours, ends)
+        assert sarlib.spread_pick(y, [t * 1e-3 for t in same_region]) == -1          # nobody elsewhere: no pair
+    # the search with 80 GiB of other allocations around: the yardstick drops to 174-175 us and the pair comes in at
+    # 0.932 of it, candidates in the same region at 0.98 and more: still two populations
+    assert sarlib.spread_pick(0.1745, [0.1761, 0.1718, 0.1810, 0.1627]) == 3
+    # two candidates elsewhere (the other two regions): the faster one
+    assert sarlib.spread_pick(0.185, [0.190, 0.160, 0.186, 0.158]) == 3
+    # populations that run into each other: a candidate at 0.94 of the yardstick with another at 0.96 right above it
+    # is not a clear verdict (the same candidate with the next one at 0.98 is)
+    assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1776]) == -1
+    assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1813]) == 1
+    assert sarlib.spread_pick(0.170, [0.1560]) == 0                                   # 0.918, alone: clear of the yardstick itself
+    assert sarlib.spread_pick(0.170, [0.1620]) == -1                                  # 0.953: not below the limit
+    # failed probes say nothing, and no candidates is no pair
+    assert sarlib.spread_pick(0.185, [-1.0, 0.0, 0.158]) == 2
+    assert sarlib.spread_pick(0.185, [-1.0]) == -1
+    assert sarlib.spread_pick(0.185, []) == -1
     # failed probes (negative) and nonsense never count as elsewhere; bad arguments are refused
     assert not sarlib.spread_is_elsewhere(0.185, -1.0)
     assert not sarlib.spread_is_elsewhere(0.185, 0.0)

@@ -88,7 +88,7 @@ def test_builtin_stragglar_is_the_table_in_the_cu(sarlib, n):
 @pytest.mark.parametrize("name,n", [("synth_pow2_n8.txt", 8), ("synth_pow2_n16.txt", 16), ("synth_pow2_n32.txt", 32),
                                     ("synth_nonpow2_n6.txt", 6), ("synth_nonpow2_n10.txt", 10),
                                     ("synth_nonpow2_n12.txt", 12), ("synth_nonpow2_n14.txt", 14),
-                                    ("synth_nonpow2_n24.txt", 24), ("synth_pow2_n8_stdout.txt", 8),
+                                    ("synth_nonpow2_n24.txt", 24), ("synth_nonpow2_n48.txt", 48), ("synth_pow2_n8_stdout.txt", 8),
                                     ("synth_nonpow2_n6_stdout.txt", 6)])
 def test_parser_reads_synthesizer_output(sarlib, name, n):
     """Tables printed by the reference synthesizers (fixtures) parse, validate and keep every move."""
@@ -102,10 +102,12 @@ def test_parser_reads_synthesizer_output(sarlib, name, n):
 
 
 def test_round_counts_match_the_reference(sarlib):
-    """n-2+log2 n for powers of two (synthesizer_pow2.py:275); 6->7, 12->15, 24->27 (simulation.py:7)."""
+    """n-2+log2 n for powers of two (synthesizer_pow2.py:275); 6->7, 12->15, 24->27 (simulation.py:7).  For 48 ranks
+    simulation.py:7 quotes 57 rounds; the reference script itself, imported under networkx 3.4.2 (the fixture's
+    header), yields 55: the count depends on how max_weight_matching breaks ties, which the reference does not pin."""
     for name, n, rounds in [("synth_pow2_n8.txt", 8, 9), ("synth_pow2_n16.txt", 16, 18), ("synth_pow2_n32.txt", 32, 35),
                             ("synth_nonpow2_n6.txt", 6, 7), ("synth_nonpow2_n12.txt", 12, 15),
-                            ("synth_nonpow2_n24.txt", 24, 27), ("stragglar_n4_cu.txt", 4, 4)]:
+                            ("synth_nonpow2_n24.txt", 24, 27), ("synth_nonpow2_n48.txt", 48, 55), ("stragglar_n4_cu.txt", 4, 4)]:
         assert sarlib.parse(read_golden(name), n).num_rounds == rounds
 
 
@@ -272,7 +274,7 @@ def test_synthesizer_pow2_n4_gives_the_table_in_the_cu():
     assert [sorted(r) for r in parse_table(text)] == [sorted(r) for r in parse_table(read_golden("stragglar_n4_cu.txt"))]
 
 
-@pytest.mark.parametrize("n", [6, 10, 12, 14, 24])
+@pytest.mark.parametrize("n", [6, 10, 12, 14, 24, 48])
 def test_synthesizer_nonpow2_reproduces_the_reference_tables(n):
     nx = pytest.importorskip("networkx")
     from stragglar_amd import synthesizer_nonpow2

@@ -4,7 +4,7 @@ on a smaller input, then a schedule with pre-work and one that needs the per-rou
 import numpy as np
 import pytest
 
-from conftest import assert_bits_equal, make_inputs, read_golden
+from conftest import assert_bits_equal, hip_runtime, make_inputs, read_golden
 
 pytestmark = pytest.mark.gpu
 
@@ -87,3 +87,109 @@ def test_static_entry_point_refuses_what_it_cannot_hold(sarlib, gpu_ctx):
         with pytest.raises(SarError) as e:
             sarlib.run_static(ptrs, (2 << 20) + 4096, "f32", sarlib.builtin("ring", 2))
         assert "shorter than bytes_per_rank" in str(e.value)
+
+
+def test_static_entry_point_allocates_no_device_memory(sarlib, gpu_ctx):
+    """What the entry point is for: free device memory reads the same before and after warm calls (the tables go into
+    the static array, not into allocations), also for a call made while this thread has a capture open on another
+    stream, which ends normally."""
+    import ctypes
+    hip = hip_runtime()
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    n = 8
+    nbytes = sarlib.pad_bytes(1 << 20, n)
+    inputs = make_inputs(n, nbytes // 4, "f32", seed=21)
+    main, pre, ring = sarlib.parse(read_golden("stragglar_n8_cu.txt"), n), sarlib.builtin("prework_rs", n), sarlib.builtin("ring", n)
+    run_stream, cap_stream = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(run_stream), 1) == 0       # hipStreamNonBlocking
+    assert hip.hipStreamCreateWithFlags(ctypes.byref(cap_stream), 1) == 0
+    with sarlib.context(0) as mem:
+        mem.alloc_ranks(n, nbytes, "f32")
+        ptrs = [mem.rank_pointer(r) for r in range(n)]
+
+        def one_call(sched, prework):
+            for r, x in enumerate(inputs):
+                mem.upload(r, x)
+            sarlib.run_static(ptrs, nbytes, "f32", sched, prework, stream=run_stream.value)
+            return [mem.download(r) for r in range(n)]
+
+        want = one_call(main, pre)                    # warm: code objects loaded, the runtime's own pools grown
+        one_call(ring, None)
+        before = free_bytes()
+        got = one_call(main, pre)
+        one_call(ring, None)
+        assert free_bytes() == before, "sar_run_static changed the free device memory"
+        for r in range(n):
+            assert_bits_equal(got[r], want[r], "second call, rank %d" % r)
+        # a capture open on another stream of this thread (thread-local mode): the call allocates nothing and is legal
+        graph = ctypes.c_void_p()
+        for r, x in enumerate(inputs):
+            mem.upload(r, x)
+        assert hip.hipStreamBeginCapture(cap_stream, 1) == 0                    # hipStreamCaptureModeThreadLocal
+        try:
+            sarlib.run_static(ptrs, nbytes, "f32", main, pre, stream=run_stream.value)
+        finally:
+            ended = hip.hipStreamEndCapture(cap_stream, ctypes.byref(graph))
+        assert ended == 0
+        if graph.value:
+            assert hip.hipGraphDestroy(graph) == 0
+        for r in range(n):
+            assert_bits_equal(mem.download(r), want[r], "call beside an open capture, rank %d" % r)
+        assert free_bytes() == before
+    assert hip.hipStreamDestroy(run_stream) == 0 and hip.hipStreamDestroy(cap_stream) == 0
+
+
+def test_static_entry_point_calls_from_two_threads_take_turns(sarlib, gpu_ctx):
+    """All calls on a GPU share the one static array; the library lets them take turns.  Two threads, each with rank
+    buffers and a stream of its own, call at the same time: every result is what a call on its own gives."""
+    import ctypes
+    import threading
+    hip = hip_runtime()
+    n = 8
+    sizes = [sarlib.pad_bytes(2 << 20, n), sarlib.pad_bytes(96 << 10, n)]
+    scheds = [(sarlib.parse(read_golden("stragglar_n8_cu.txt"), n), sarlib.builtin("prework_rs", n)), (sarlib.builtin("rhd", n), None)]
+    mems, ptrs, inputs, want, streams = [], [], [], [], []
+    try:
+        for k in range(2):
+            mem = sarlib.context(0)
+            mems.append(mem)
+            mem.alloc_ranks(n, sizes[k], "f32")
+            ptrs.append([mem.rank_pointer(r) for r in range(n)])
+            inputs.append(make_inputs(n, sizes[k] // 4, "f32", seed=31 + k))
+            for r, x in enumerate(inputs[k]):
+                mem.upload(r, x)
+            sarlib.run_static(ptrs[k], sizes[k], "f32", scheds[k][0], scheds[k][1])
+            want.append([mem.download(r) for r in range(n)])
+            st = ctypes.c_void_p()
+            assert hip.hipStreamCreateWithFlags(ctypes.byref(st), 1) == 0
+            streams.append(st)
+        errors = []
+
+        def worker(k):
+            try:
+                for it in range(6):
+                    for r, x in enumerate(inputs[k]):
+                        mems[k].upload(r, x)
+                    sarlib.run_static(ptrs[k], sizes[k], "f32", scheds[k][0], scheds[k][1], stream=streams[k].value)
+                    for r in range(n):
+                        assert_bits_equal(mems[k].download(r), want[k][r], "thread %d call %d rank %d" % (k, it, r))
+            except BaseException as e:      # noqa: BLE001 -- reported by the main thread
+                errors.append(e)
+
+        threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(120)
+        assert not any(t.is_alive() for t in threads)
+        assert not errors, errors
+    finally:
+        for st in streams:
+            hip.hipStreamDestroy(st)
+        for mem in mems:
+            mem.close()
