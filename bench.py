@@ -185,19 +185,20 @@ def leg_rates(st, ms, fused=False):
     """Memory-side and algorithmic rates of one leg; `fused`: pre-work and schedule ran as the one launch."""
     alg = st.algorithmic_bytes + (st.prework_bytes if fused else 0)
     mem = alg - (st.fused_forwarded_bytes + st.fused_elided_store_bytes if fused else st.forwarded_bytes + st.elided_store_bytes)
-    return {"ms_per_step": round(ms, 5), "memory_bytes_per_step": int(mem), "memory_side_GBps": round(mem / ms / 1e6, 1),
-            "frac_of_hbm_peak": round(mem / ms / 1e6 / HBM_PEAK_GBPS, 4), "algorithmic_bytes_per_step": int(alg),
+    return {"ms": round(ms, 5), "memory_bytes": int(mem), "GBps": round(mem / ms / 1e6, 1), "frac": round(mem / ms / 1e6 / HBM_PEAK_GBPS, 4),
             "algorithmic_GBps": round(alg / ms / 1e6, 1)}
 
 
 def other_configs(lib, ctx, orc, many, steps, warmup):
-    """The BASELINE configurations beside the headline one, each timed by this run on the same device, same step
-    protocol (inputs restored from the device snapshot before every step, untimed; events on the executor's stream):
-    what the reference binary times for any size, algorithm and delay (allreduce_8GPU.cu:1009-1066,
-    reducescatter.cu:88-121).  Results are checked against the CPU checker on whole buffers when it is loaded."""
+    """The BASELINE configurations beside the headline one, each timed by this run on the same device with the same
+    step protocol (inputs restored from the device snapshot before every step, untimed; events on the executor's
+    stream): what the reference binary times for any size, algorithm and delay (allreduce_8GPU.cu:1009-1066,
+    reducescatter.cu:88-121).  GBps / frac: bytes that reach memory per step / mean step time, and its share of the
+    8 TB/s peak; algorithmic_GBps: every row priced on its own.  ok: all ranks hold the same bits afterwards and, with the
+    CPU checker loaded, every element of every rank equals the checker's (null when a check was not made)."""
     import numpy as np
     from oracle import parse_table
-    out = {}
+    out = {"keys": "ms = mean step, GBps/frac = bytes that reach memory / ms (of 8 TB/s), ok = ranks identical and every element equal to the CPU checker's"}
 
     def table(n):
         path = os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)
@@ -220,21 +221,19 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
             ctx.restore(); ts.append(ctx.run(delay))
         return ts
 
-    def check(alg, rounds, dtype, delay, n, parts):
-        """ranks identical on the device, and every element of every rank against the CPU checker."""
-        res = {"ranks_identical_after_run": bool(ctx.ranks_identical((ctx.elems // parts) * parts))}
-        if orc is not None:
-            ctx.restore()
-            want = [ctx.download(r) for r in range(n)]
-            orc.set_threads(many)
-            orc.run(alg, want, dtype, rounds=rounds, delay=delay)
-            orc.set_threads(1)
-            ctx.restore(); ctx.run(delay)
-            ok = True
-            for r in range(n):
-                ok = ok and np.array_equal(ctx.download(r).view(np.uint8), want[r].view(np.uint8))
-            res["bit_exact_vs_cpu_checker"] = bool(ok)
-        return res
+    def ok(alg, rounds, dtype, delay, n, parts):
+        same = bool(ctx.ranks_identical((ctx.elems // parts) * parts))
+        if orc is None:
+            return same and None
+        ctx.restore()
+        want = [ctx.download(r) for r in range(n)]
+        orc.set_threads(many)
+        orc.run(alg, want, dtype, rounds=rounds, delay=delay)
+        orc.set_threads(1)
+        ctx.restore(); ctx.run(delay)
+        for r in range(n):
+            same = same and np.array_equal(ctx.download(r).view(np.uint8), want[r].view(np.uint8))
+        return bool(same)
 
     # configs[0]: n = 4, 1 MiB fp32 per rank; the ReduceScatter pre-work materialised (the data are random, so "pre-work
     # done" cannot be pre-filled): pre-work and the four rounds as the one launch sar_run(0) makes of them
@@ -246,10 +245,9 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     st = ctx.stats()
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
-    leg.update({"workload": "n=4 stragglar, %d B fp32 per rank, uniform[-1,1), ReduceScatter pre-work + 4 rounds" % nbytes,
-                "ms_per_step_min": round(min(ts), 5), "launches": int(st.launches) if not st.fused_prework else 1,
-                "note": "fits the caches: a launch-latency figure, not an HBM rate"})
-    leg.update(check("stragglar", rounds4, "f32", 0.0, n, n - 1))
+    leg.update({"what": "n=4 stragglar, %d B fp32 per rank, pre-work + 4 rounds; fits the caches: a latency figure" % nbytes,
+                "us_min": round(min(ts) * 1e3, 2), "launches": 1 if st.fused_prework else int(st.launches),
+                "ok": ok("stragglar", rounds4, "f32", 0.0, n, n - 1)})
     out["config0_n4_1MiB_f32"] = leg
 
     # configs[3]: n = 6 (synthesizer_nonpow2 6), 64 MiB fp16 per rank padded as pad_buffers.py, uniform[-0.5,0.5),
@@ -262,33 +260,28 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     st = ctx.stats()
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
-    leg.update({"workload": "n=6 stragglar (non-power-of-two table), %d B fp16 per rank, uniform[-0.5,0.5), ReduceScatter pre-work + 7 rounds" % nbytes,
-                "ms_per_step_min": round(min(ts), 5), "pre_work_in_the_same_launch": bool(st.fused_prework)})
-    leg.update(check("stragglar", rounds6, "f16", 0.0, n, n - 1))
+    leg.update({"what": "n=6 stragglar (non-power-of-two table), %d B fp16 per rank, pre-work + 7 rounds" % nbytes,
+                "launches": 1 if st.fused_prework else int(st.launches), "ok": ok("stragglar", rounds6, "f16", 0.0, n, n - 1)})
     out["config3_n6_64MiB_f16_prework"] = leg
 
     # configs[4]: message sizes for n = 8 fp32, four algorithms, eager launches
     n = 8
     main8, rounds8 = table(n)
-    sweep = {}
+    sweep = {"columns": ["us", "GBps", "frac", "ok"],
+             "note": "eager launches; 16 MiB per rank and below fit the 256 MB Infinity Cache: launch latency and caches, not HBM"}
     for label, raw in (("4KiB", 4 << 10), ("64KiB", 64 << 10), ("1MiB", 1 << 20), ("16MiB", 16 << 20), ("256MiB", 256 << 20), ("1GiB", 1 << 30)):
         nbytes = lib.pad_bytes(raw, n)
         place(n, nbytes, "f32", lambda r: ctx.fill_uniform(r, 500 + r, -1.0, 1.0))
         k, w = (steps, warmup) if raw <= (256 << 20) else (max(3, steps // 4), 1)
-        row = {"bytes_per_rank": nbytes}
+        row = {}
         for alg in ("stragglar", "ring", "rhd", "direct"):
             sched = main8 if alg == "stragglar" else lib.builtin(alg, n)
             ctx.prepare(sched, None)
             st = ctx.stats()
-            ts = steps_ms(-1.0, k, w)
-            leg = leg_rates(st, statistics.fmean(ts))
-            leg.update({"ms_per_step_min": round(min(ts), 5), "us_per_step": round(statistics.fmean(ts) * 1e3, 2), "launches": int(st.launches),
-                        "executor_used": "column" if st.executor == 1 else "rounds"})
-            leg.update(check(alg, rounds8 if alg == "stragglar" else None, "f32", -1.0, n, sched.parts))
-            row[alg] = leg
+            r = leg_rates(st, statistics.fmean(steps_ms(-1.0, k, w)))
+            row[alg] = [round(r["ms"] * 1e3, 2), r["GBps"], r["frac"], ok(alg, rounds8 if alg == "stragglar" else None, "f32", -1.0, n, sched.parts)]
         sweep[label] = row
-    sweep["note"] = "16 MiB per rank and below fit the 256 MB Infinity Cache: those rows measure launch latency and caches, not HBM"
-    out["config4_message_sizes_n8_f32"] = sweep
+    out["config4_sizes_n8_f32"] = sweep
 
     # configs[2]: n = 8, 1 GiB bf16 per rank, normal(0, 1e-3), sums in bf16; the straggler arrives DELAY = 5 ms late
     # while ranks 0-6 do their ReduceScatter pre-work (allreduce_8GPU.cu:876-898)
@@ -298,13 +291,12 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     pre8 = lib.builtin("prework_rs", n)
     k, w = max(3, steps // 4), 1
     ctx.prepare(main8, pre8)
-    st = ctx.stats()
     ts = steps_ms(delay, k, w)
     total = statistics.fmean(ts)
-    leg = {"workload": "n=8 stragglar, %d B bf16 per rank, normal(0, 1e-3), DELAY = %.0f ms: pre-work on a second stream beside the straggler's sleep" % (nbytes, delay),
-           "ms_per_step": round(total, 5), "ms_per_step_min": round(min(ts), 5), "ms_after_the_stragglers_arrival": round(total - delay, 5),
-           "reference_style_GiBps": round(nbytes / 2.0 ** 30 * 1000.0 / (total - delay), 2)}
-    leg.update(check("stragglar", rounds8, "bf16", delay, n, n - 1))
+    leg = {"what": "n=8 stragglar, %d B bf16 per rank, normal(0, 1e-3), DELAY = %.0f ms: pre-work on a second stream beside the straggler's sleep" % (nbytes, delay),
+           "ms": round(total, 5), "ms_after_arrival": round(total - delay, 5),
+           "reference_style_GiBps": round(nbytes / 2.0 ** 30 * 1000.0 / (total - delay), 2),
+           "ok": ok("stragglar", rounds8, "bf16", delay, n, n - 1)}
     # the two kernels of that run, each on its own: bytes that reach memory / time of the launch
     ctx.prepare(main8, None)
     st = ctx.stats()
@@ -314,9 +306,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     leg["schedule_kernel"] = leg_rates(st, statistics.fmean(kms[w:]))
     ctx.prepare(pre8, None)
     st = ctx.stats()
-    ts = steps_ms(-1.0, k, w)
-    leg["prework_kernel"] = leg_rates(st, statistics.fmean(ts))
-    leg["prework_kernel"]["rows"] = "7 multi-source rows: 7 chunks read, 1 written per chunk index"
+    leg["prework_kernel"] = leg_rates(st, statistics.fmean(steps_ms(-1.0, k, w)))
     out["config2_n8_1GiB_bf16_delay5ms"] = leg
     return out
 
@@ -580,7 +570,7 @@ def main():
                 leg["bit_exact_vs_cpu_checker"] = bool(bit_exact(alg, None))
             comps[alg] = leg
         rec["comparators"] = comps
-    if not args.no_other_configs and not args.no_comparators and args.alg == "stragglar" and n == 8 and not args.graph and not overrides:
+    if not args.no_other_configs and not args.no_comparators and args.alg == "stragglar" and n == 8 and args.mib == 256 and not args.graph and not overrides:
         t0 = time.perf_counter()
         rec["other_configs"] = other_configs(lib, ctx, orc, many, args.steps, args.warmup)
         rec["other_configs"]["seconds"] = round(time.perf_counter() - t0, 1)
@@ -592,8 +582,8 @@ def main():
 
     def failed(node):
         if isinstance(node, dict):
-            return node.get("ranks_identical_after_run") is False or node.get("bit_exact_vs_cpu_checker") is False or any(failed(v) for v in node.values())
-        return False
+            return node.get("ok") is False or any(failed(v) for v in node.values())
+        return isinstance(node, list) and len(node) == 4 and node[3] is False
     bad = bad or failed(rec.get("other_configs", {}))
     if bad:
         sys.exit(1)

@@ -104,6 +104,7 @@ typedef struct sar_stats_t {
     float spread_same_ms;          /* probed, the region probe's time for two windows in one region (the fastest  */
     float spread_pair_ms;          /* of four pairs) and for the pair that was kept (the slower of its two probes), and */
     uint64_t spread_search_bytes;  /* the most device memory held at a time while looking, the pair included      */
+                                   /* (the search is the GPU's, shared: whichever context ran it last)            */
     uint64_t fused_forwarded_bytes;    /* the same two figures for the single launch of pre-work + main schedule  */
     uint64_t fused_elided_store_bytes; /* (fused_prework = 1), out of algorithmic_bytes + prework_bytes           */
     uint64_t placed_pool_bytes;    /* the GPU's pair of allocations in different regions of HBM, shared by all     */
@@ -170,10 +171,11 @@ typedef struct sar_tuning_t {
                           /*     MiB, plans whose value slots limit the workgroups per CU;           */
                           /*     2 = in every plan; 0 = never                                        */
     int32_t arena_spread; /* sar_alloc_ranks: 1 = for payloads of 128 MiB and more, half the ranks go   */
-                          /*     into an allocation of their own that a short timing probe has shown */
-                          /*     to lie in another region of HBM than the first half's (MI355X:     */
-                          /*     buffers in different thirds of the 288 GiB disturb each other less; */
-                          /*     the pair is kept for the life of the context); ranks back to back  */
+                          /*     into an allocation that a short timing probe has shown to lie in    */
+                          /*     another region of HBM than the first half's (MI355X: buffers in     */
+                          /*     different thirds of the 288 GiB disturb each other less).  The two  */
+                          /*     allocations are ONE pair per GPU and process, shared by all contexts */
+                          /*     and released with the last context that used it; ranks back to back */
                           /*     when no such pair is found or the device lacks the room; 0 = never  */
     int32_t col_prework;  /* 1 = multi-source rows run in the column kernel as well: the pre-work that      */
                           /*     overlaps the straggler's delay is one column launch on the second stream,  */
@@ -263,8 +265,8 @@ void sar_destroy(sar_ctx* ctx);
 /* Rank buffers, replacing cudaMallocAsync(d_buffers[i]) (allreduce_8GPU.cu
  * :977-990).  No temp buffers exist: exchanges are fused.  All ranks share one
  * arena; rank r starts at r*stride, stride = bytes rounded up to 2 MiB (with
- * tuning.arena_spread the upper half of the ranks starts over in a second
- * allocation).  bytes_per_rank: a positive multiple of the element size, at
+ * tuning.arena_spread the upper half of the ranks starts over in the second
+ * of the GPU's two placed allocations).  bytes_per_rank: a positive multiple of the element size, at
  * most SAR_MAX_RANK_BYTES. */
 int sar_alloc_ranks(sar_ctx* ctx, int n, uint64_t bytes_per_rank, int dtype);
 
@@ -288,8 +290,9 @@ int sar_rank_pointer(sar_ctx* ctx, int rank, void** device_ptr);
  * different regions of HBM (the search sar_alloc_ranks uses) and are mapped next to each other, which rows of an
  * ordinary allocation cannot have; *placed says whether (may be null), *reason why not (SAR_SPREAD_*, may be null).
  * Otherwise a plain allocation.  The rows belong to the context: valid until the next sar_alloc_rows, sar_free_rows
- * or sar_destroy; rank buffers adopted from them are dropped with them.  A placed pair (2 x 8 GiB, more for larger
- * halves) stays with the context after sar_free_rows for the next call. */
+ * or sar_destroy; rank buffers adopted from them are dropped with them.  The two allocations are the GPU's one pair
+ * that all contexts of the process share (see sar_alloc_ranks); the rows take the place across its junction, which
+ * one block of rows can hold at a time (a second one is a plain allocation, reason SAR_SPREAD_POOL_BUSY). */
 int sar_alloc_rows(sar_ctx* ctx, int n, uint64_t bytes_per_row, void** base, int* placed, int* reason);
 int sar_free_rows(sar_ctx* ctx);
 
@@ -347,10 +350,12 @@ int sar_run(sar_ctx* ctx, float delay_ms, float* elapsed_ms);
  * tables take a few KiB, a 64-rank ring about half a MiB).  `stream` is the caller's hipStream_t (NULL = the
  * null stream): the tables are copied and the kernels launched on it, and the call returns when it has drained
  * and the result is complete (so `stream` itself must not be capturing: the call is for a process that has a
- * capture open elsewhere, or may not allocate for other reasons; the table copies are hipMemcpyAsync from
- * ordinary host memory, staged by the runtime).  device_ptrs as for sar_adopt_ranks (checked the same way); the default tuning
+ * capture open elsewhere, or may not allocate for other reasons; the calling thread runs in relaxed capture mode
+ * for the duration of the call, since thread-local and global mode refuse hipStreamSynchronize on any stream; the
+ * table copies are hipMemcpyAsync from ordinary host memory, staged by the runtime).  device_ptrs as for sar_adopt_ranks (checked the same way); the default tuning
  * applies.  No context is needed or touched.  All calls on one GPU share the one array, which keeps the last
- * call's tables: calls that overlap in time on the same GPU race and must be serialised by the caller. */
+ * call's tables; the library lets them take turns (a per-GPU lock held from the first table copy until the stream
+ * has drained), so calls from several threads are safe and run one after the other. */
 int sar_run_static(int device, void* stream, const sar_schedule* prework, const sar_schedule* main_sched, int n,
                    void* const* device_ptrs, uint64_t bytes_per_rank, int dtype);
 uint64_t sar_static_scratch_bytes(void);

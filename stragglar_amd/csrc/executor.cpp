@@ -1461,8 +1461,15 @@ int run_static_body(int device, void* stream, const sar_schedule* prework, const
         }
         return SAR_OK;
     };
+    // The caller may have a stream capture open in this thread, or another thread one in global mode: both refuse
+    // "potentially unsafe" calls, hipStreamSynchronize among them, also on streams that are not being captured.
+    // Nothing here touches a capturing stream (`st` must not be one), so the thread takes relaxed mode for the call.
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool relaxed = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    if (!relaxed) (void)hipGetLastError();
     rc = enqueue();
     const hipError_t drained = hipStreamSynchronize(st);
+    if (relaxed) (void)hipThreadExchangeStreamCaptureMode(&mode);
     if (rc != SAR_OK) return rc;
     if (drained != hipSuccess) return set_error(SAR_EHIP, std::string("hipStreamSynchronize: ") + hipGetErrorString(drained));
     return SAR_OK;

@@ -8,16 +8,20 @@ For every size (bytes per rank before padding; padded as pad_buffers.py pads) an
 as the reference's benchmark runs it with DELAY = -1 (allreduce_8GPU.cu:1029-1047: the same four algorithms at any
 size), the inputs restored before every iteration, eagerly launched and as a replayed hipGraph.  One CSV line each:
 
-    algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps
+    algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps,host_call_us
 
 memory_GBps counts the bytes the plan sends to memory (operands taken from LDS slots and stores that are left out do
 not count), algorithmic_GBps prices every row on its own.  Below about 16 MiB per rank (n = 8) the rank buffers stay in
-the caches and the memory figure is not an HBM rate.
+the caches and the memory figure is not an HBM rate.  median_us / min_us are the time between the two events sar_run
+records around its launches; host_call_us is the median time the sar_run call itself takes on the host clock (event
+records, the launch or graph launch, the wait for the stop event, the binding's overhead): at small sizes the difference
+between the eager and the graph line is what a graph launch costs the host more than a kernel launch.
 """
 import argparse
 import os
 import statistics
 import sys
+import time
 
 from . import capi
 
@@ -35,7 +39,7 @@ def main(argv=None) -> int:
     lib = capi.load_library()
     n = args.ranks
     ctx = lib.context(0)
-    print("algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps")
+    print("algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps,host_call_us")
     for raw in [int(x) for x in args.sizes.split(",") if x]:
         nbytes = lib.pad_bytes(raw, n)
         ctx.alloc_ranks(n, nbytes, args.dtype)
@@ -53,16 +57,20 @@ def main(argv=None) -> int:
             for graph in (0, 1):
                 ctx.prepare(sched, None, use_graph=bool(graph))
                 st = ctx.stats()
-                ts = []
+                ts, host = [], []
                 for it in range(args.iters + 2):
                     ctx.restore()
+                    t0 = time.perf_counter()
                     ms = ctx.run(-1.0)
+                    t1 = time.perf_counter()
                     if it >= 2:
                         ts.append(ms)
+                        host.append(t1 - t0)
                 med = statistics.median(ts)
                 to_memory = st.algorithmic_bytes - st.forwarded_bytes - st.elided_store_bytes
-                print("%s,%d,%d,%d,%s,%.2f,%.2f,%.0f,%.0f" % (alg, nbytes, graph, st.launches, "column" if st.executor else "rounds",
-                                                             med * 1e3, min(ts) * 1e3, to_memory / med / 1e6, st.algorithmic_bytes / med / 1e6), flush=True)
+                print("%s,%d,%d,%d,%s,%.2f,%.2f,%.0f,%.0f,%.1f" % (alg, nbytes, graph, st.launches, "column" if st.executor else "rounds",
+                                                                  med * 1e3, min(ts) * 1e3, to_memory / med / 1e6, st.algorithmic_bytes / med / 1e6,
+                                                                  statistics.median(host) * 1e6), flush=True)
     ctx.close()
     return 0
 

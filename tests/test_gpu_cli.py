@@ -189,8 +189,9 @@ def test_size_sweep_tool():
     p = run(sys.executable, "-m", "stragglar_amd.size_sweep", "--sizes", "4096,1048576", "--iters", "3")
     assert p.returncode == 0, p.stdout + p.stderr
     lines = p.stdout.splitlines()
-    assert lines[0] == "algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps"
+    assert lines[0] == "algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps,host_call_us"
     rows = [l.split(",") for l in lines[1:]]
+    assert all(float(r[9]) > float(r[6]) for r in rows)          # the call on the host clock contains the span between its two events
     assert len(rows) == 2 * 4 * 2 and {r[0] for r in rows} == {"stragglar", "ring", "rhd", "direct"}
     assert {int(r[1]) for r in rows} == {7168, 1053696} and all(float(r[5]) >= float(r[6]) > 0 for r in rows)
 
@@ -257,6 +258,36 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
         assert rec["bit_exact_vs_cpu_checker"] is True
 
 
+def test_bench_default_workload_carries_every_baseline_config():
+    """The run the harness makes (the default workload, here with few steps): besides the headline line the other
+    BASELINE configurations are timed and checked in the same run -- n=4 1 MiB, n=6 fp16 with pre-work, the message-size
+    sweep of the four algorithms up to 1 GiB per rank, bf16 1 GiB with DELAY = 5 ms and its two kernels."""
+    import json
+    import sys
+    p = run(sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "4", "--warmup", "1", "--cpu-seconds", "0.5", "--no-live-traffic")
+    assert p.returncode == 0, p.stdout[-2000:] + p.stderr[-2000:]
+    lines = [l for l in p.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    other = rec["other_configs"]
+    assert sorted(k for k in other if k.startswith("config")) == ["config0_n4_1MiB_f32", "config2_n8_1GiB_bf16_delay5ms", "config3_n6_64MiB_f16_prework", "config4_sizes_n8_f32"]
+    assert other["config0_n4_1MiB_f32"]["ok"] is True and other["config0_n4_1MiB_f32"]["launches"] == 1
+    c3 = other["config3_n6_64MiB_f16_prework"]
+    # pre-work + table in one launch: 30 chunks read and 30 written (C = S / 5): the pre-work's result is never stored
+    assert c3["ok"] is True and c3["launches"] == 1 and abs(c3["memory_bytes"] - 12 * 67112960) <= 67112960 // 100
+    sweep = other["config4_sizes_n8_f32"]
+    for size in ("4KiB", "64KiB", "1MiB", "16MiB", "256MiB", "1GiB"):
+        assert sorted(sweep[size]) == ["direct", "rhd", "ring", "stragglar"]
+        for us, gbps, frac, ok in sweep[size].values():
+            assert us > 0 and gbps > 0 and ok is True
+    assert sweep["1GiB"]["stragglar"][2] > 0.5                                                  # an HBM rate at this size
+    c2 = other["config2_n8_1GiB_bf16_delay5ms"]
+    assert c2["ok"] is True and c2["ms"] > 5.0 and 0 < c2["ms_after_arrival"] < 5.0
+    assert c2["schedule_kernel"]["memory_bytes"] == 10 * 1073744896 and c2["prework_kernel"]["memory_bytes"] == 8 * 1073744896
+    assert 0.5 < c2["schedule_kernel"]["frac"] < 1.0 and 0.5 < c2["prework_kernel"]["frac"] < 1.0
+    assert other["seconds"] < 150
+
+
 def test_bench_refuses_more_than_one_gpu():
     import sys
     p = run(sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2")
@@ -268,3 +299,28 @@ def test_smoke_entry_point():
     import sys
     p = run(sys.executable, "-c", "import sys; sys.path.insert(0, %r); import __graft_entry__ as g; g.smoke()" % ROOT)
     assert p.returncode == 0 and "smoke ok" in p.stdout, p.stdout + p.stderr
+
+
+def test_tuning_sweep_and_placement_mixes_tools():
+    """The two measurement tools behind the tracked experiment records: one schedule under a grid of tunings, and the
+    schedules' stream mixes laid over the regions of HBM in different ways (here on a small allocation: the tool must
+    say so when it finds no two regions in it, and must not fail otherwise)."""
+    import sys
+    p = run(sys.executable, "-m", "stragglar_amd.tuning_sweep", "--alg", "ring", "--ranks", "8", "--mib", "4", "--iters", "3",
+            "--vary", "col_fuse_copies=1,2", "--vary", "col_block=0,256")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = [l for l in p.stdout.splitlines() if not l.startswith("#")]
+    assert lines[0].startswith("col_fuse_copies,col_block,executor,col_block,col_slots,median_us,min_us,memory_bytes,memory_GBps")
+    rows = [l.split(",") for l in lines[1:]]
+    assert [(r[0], r[1]) for r in rows] == [("1", "0"), ("1", "256"), ("2", "0"), ("2", "256")]
+    assert all(r[-1] == "True" and float(r[5]) >= float(r[6]) > 0 for r in rows)
+    p = run(sys.executable, "-m", "stragglar_amd.tuning_sweep", "--schedule", os.path.join(ROOT, "stragglar_amd", "schedules", "exchanges_n8.rows"),
+            "--mib", "4", "--iters", "3", "--vary", "cache_policy=2,1")
+    assert p.returncode == 0 and len([l for l in p.stdout.splitlines() if l.startswith(("2,", "1,"))]) == 2, p.stdout + p.stderr
+    assert run(sys.executable, "-m", "stragglar_amd.tuning_sweep", "--vary", "no_such_field=1").returncode == 2
+    p = run(sys.executable, "-m", "stragglar_amd.hbm_regions", "--mixes", "--gib", "32", "--slot-gib", "1", "--per-rank-mib", "64", "--stream-mib", "64")
+    assert p.returncode in (0, 1), p.stdout + p.stderr
+    if p.returncode == 1:
+        assert "no two regions" in p.stderr
+    else:
+        assert "pre-work" in p.stdout and "exchanges" in p.stdout and "ring" in p.stdout
