@@ -612,6 +612,67 @@ def test_placed_memory_comes_back(sarlib, gpu_ctx):
     assert min(abs(after[0] - start), abs(after[0] - (start - pool_bytes))) <= slack, (start - after[0], pool_bytes)
 
 
+def test_contexts_share_the_placed_pair(sarlib, gpu_ctx, oracle):
+    """Three contexts hold rank arenas on the GPU's one pair of placed allocations at the same time, and rows across its
+    junction: leases do not overlap, every context computes the checker's bits whatever its neighbours do, the place
+    across the junction goes to one block of rows at a time, and leases come back when their holders let go."""
+    n, dtype = 8, "f32"
+    table = read_golden("stragglar_n8_cu.txt")
+    sizes = [7 * 8 * 90000 * 4, 7 * 8 * 150000 * 4, 7 * 8 * 70000 * 4]            # 20, 34 and 16 MB per rank: 128 MiB and more in all
+    ctxs = [sarlib.context(0) for _ in sizes]
+    try:
+        ins, wants, spans = [], [], []
+        for c, nbytes in zip(ctxs, sizes):
+            c.alloc_ranks(n, nbytes, dtype)
+            x = make_inputs(n, nbytes // 4, dtype, seed=nbytes % 1013)
+            for r in range(n):
+                c.upload(r, x[r])
+            ins.append(x)
+            wants.append(run_oracle(oracle, "stragglar", x, dtype, table, delay=0.0))
+            spans += [(c.rank_pointer(r), c.rank_pointer(r) + nbytes) for r in range(n)]
+            c.prepare(sarlib.parse(table, n), sarlib.builtin("prework_rs", n))
+        spans.sort()
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), "rank buffers of different contexts overlap"
+        stats = [c.stats() for c in ctxs]
+        placed = [st.spread_reason == 0 for st in stats]
+        report_placement("three contexts at once", stats[0])
+        if all(placed):
+            assert len({(st.placed_pool_bytes, st.spread_candidates, st.spread_same_ms, st.spread_pair_ms) for st in stats}) == 1     # one pair, one search
+            assert stats[2].placed_pool_contexts >= 3
+        for c in reversed(ctxs):                                        # all launched before any result is read
+            c.run(0.0)
+        for c, want in zip(ctxs, wants):
+            for r in range(n):
+                assert_bits_equal(c.download(r), want[r], "rank %d" % r)
+        # rows across the junction: one block at a time
+        row_bytes = 24 << 20
+        base0, placed0, reason0 = ctxs[0].alloc_rows(n, row_bytes)
+        base1, placed1, reason1 = ctxs[1].alloc_rows(n, row_bytes)
+        assert placed0 == (reason0 == 0) and placed1 == (reason1 == 0)
+        if placed0:
+            assert not placed1 and reason1 == 8                         # SAR_SPREAD_POOL_BUSY: a plain allocation instead
+            ctxs[0].free_rows()
+            base1, placed1, reason1 = ctxs[1].alloc_rows(n, row_bytes)
+            assert placed1 and reason1 == 0
+        # a context that goes takes its leases along; the others are not disturbed
+        ctxs[1].close()
+        for k in (0, 2):
+            for r in range(n):
+                ctxs[k].upload(r, ins[k][r])
+            ctxs[k].run(0.0)
+            for r in range(n):
+                assert_bits_equal(ctxs[k].download(r), wants[k][r], "after a neighbour closed, rank %d" % r)
+        if all(placed):
+            fresh = sarlib.context(0)
+            ctxs.append(fresh)
+            fresh.alloc_ranks(n, sizes[1], dtype)                        # finds room where the closed context was
+            fresh.prepare(sarlib.builtin("ring", n))
+            assert fresh.stats().spread_reason == 0
+    finally:
+        for c in ctxs:
+            c.close()
+
+
 def rows_checks(ctx, sarlib, oracle):
     import stragglar_amd as sa
     n, dtype = 8, "f32"
