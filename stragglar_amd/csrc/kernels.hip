@@ -821,8 +821,8 @@ hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t
     return hipGetLastError();
 }
 // Region probe: four write streams in window a and four in window b, stream_bytes each, all running at once.
-// How long it takes tells whether the two windows lie in the same region of HBM (see find_spread_pair in
-// executor.cpp).  The kernel times itself on the device's constant-rate wall clock -- stamps[0] = earliest start,
+// How long it takes tells whether the two windows lie in the same region of HBM (see find_pair in
+// placed_pool.cpp).  The kernel times itself on the device's constant-rate wall clock -- stamps[0] = earliest start,
 // stamps[1] = latest end with all stores acknowledged, preset by the host to ~0 and 0 -- so that neither launch
 // overhead nor a profiler's bookkeeping enters the figure.
 __global__ __launch_bounds__(256) void region_probe_kernel(char* a, char* b, uint64_t stream_bytes, unsigned long long* stamps) {
