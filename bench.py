@@ -101,8 +101,7 @@ def cpu_baseline(orc, inputs, n, elems, rounds, algorithmic_bytes, budget_s=25.0
             "sample": "%d full pass(es) of the same workload (n=%d, %d fp32 elements per rank), %.1f s of CPU work, best pass %.2f s"
                       % (len(times), n, elems, sum(times), best),
         }
-    out["cpu_baseline_multithread"]["note"] = ("threads = min(CPUs in the affinity mask, %d): a one-GPU job on this pool is granted %d host CPUs "
-                                               "whatever the machine has" % (CPU_SHARE, CPU_SHARE))
+    out["cpu_baseline_multithread"]["note"] = "threads = min(CPUs in the affinity mask, %d)" % CPU_SHARE
     orc.set_threads(1)
     return out, bufs
 
@@ -198,7 +197,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     CPU checker loaded, every element of every rank equals the checker's (null when a check was not made)."""
     import numpy as np
     from oracle import parse_table
-    out = {"keys": "ms = mean step, GBps/frac = bytes that reach memory / ms (of 8 TB/s), ok = ranks identical and every element equal to the CPU checker's"}
+    out = {"legend": "ms: mean step; GBps, frac: bytes that reach memory / ms, of 8 TB/s; ok: ranks identical and every element = CPU checker"}
 
     def table(n):
         path = os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)
@@ -245,8 +244,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     st = ctx.stats()
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
-    leg.update({"what": "n=4 stragglar, %d B fp32 per rank, pre-work + 4 rounds; fits the caches: a latency figure" % nbytes,
-                "us_min": round(min(ts) * 1e3, 2), "launches": 1 if st.fused_prework else int(st.launches),
+    leg.update({"what": "pre-work + 4 rounds, %d B per rank: fits the caches, a latency figure" % nbytes, "us_min": round(min(ts) * 1e3, 2), "launches": 1 if st.fused_prework else int(st.launches),
                 "ok": ok("stragglar", rounds4, "f32", 0.0, n, n - 1)})
     out["config0_n4_1MiB_f32"] = leg
 
@@ -260,7 +258,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     st = ctx.stats()
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
-    leg.update({"what": "n=6 stragglar (non-power-of-two table), %d B fp16 per rank, pre-work + 7 rounds" % nbytes,
+    leg.update({"what": "pre-work + 7 rounds, %d B per rank" % nbytes,
                 "launches": 1 if st.fused_prework else int(st.launches), "ok": ok("stragglar", rounds6, "f16", 0.0, n, n - 1)})
     out["config3_n6_64MiB_f16_prework"] = leg
 
@@ -268,7 +266,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     n = 8
     main8, rounds8 = table(n)
     sweep = {"columns": ["us", "GBps", "frac", "ok"],
-             "note": "eager launches; 16 MiB per rank and below fit the 256 MB Infinity Cache: launch latency and caches, not HBM"}
+             "note": "eager; <= 16 MiB per rank fits the 256 MB Infinity Cache: latency and caches, not HBM"}
     for label, raw in (("4KiB", 4 << 10), ("64KiB", 64 << 10), ("1MiB", 1 << 20), ("16MiB", 16 << 20), ("256MiB", 256 << 20), ("1GiB", 1 << 30)):
         nbytes = lib.pad_bytes(raw, n)
         place(n, nbytes, "f32", lambda r: ctx.fill_uniform(r, 500 + r, -1.0, 1.0))
@@ -293,7 +291,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     ctx.prepare(main8, pre8)
     ts = steps_ms(delay, k, w)
     total = statistics.fmean(ts)
-    leg = {"what": "n=8 stragglar, %d B bf16 per rank, normal(0, 1e-3), DELAY = %.0f ms: pre-work on a second stream beside the straggler's sleep" % (nbytes, delay),
+    leg = {"what": "%d B per rank, DELAY %.0f ms, pre-work beside the straggler's sleep" % (nbytes, delay),
            "ms": round(total, 5), "ms_after_arrival": round(total - delay, 5),
            "reference_style_GiBps": round(nbytes / 2.0 ** 30 * 1000.0 / (total - delay), 2),
            "ok": ok("stragglar", rounds8, "bf16", delay, n, n - 1)}
@@ -439,7 +437,8 @@ def main():
         "config": {"workload": "configs[1]: n=%d %s (%s), %d MiB fp32 per rank padded to %d B, uniform[-1,1) seeded per rank, "
                                "DELAY=-1, %d ranks resident in one GPU's HBM; value = bytes that reach memory per step / step time "
                                "(an HBM rate; the rows' algorithmic bytes / step time is algorithmic_GBps)" % (n, args.alg, table_name, args.mib, nbytes, n),
-                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph), "tuning": tune, "executor_used": "column" if st.executor == 1 else "rounds"},
+                   "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph),
+                   "tuning": "library defaults" if tune == lib.default_tuning().as_dict() else tune, "executor_used": "column" if st.executor == 1 else "rounds"},
         "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
         "memory_bytes_per_step": int(to_memory),
         "algorithmic_bytes_per_step": int(st.algorithmic_bytes),
