@@ -6,8 +6,10 @@ buffers of 256 MiB fp32 (padded as pad_buffers.py does: 268 441 600 B) that
 are resident in HBM, uniform[-1,1) seeded per rank, pre-work taken as done
 (DELAY = -1 semantics).  Inputs are restored from a device-side snapshot
 before every step, outside the timed region, as the reference re-fills before
-every iteration; each step is timed with HIP events on the executor's stream,
-as the reference times each iteration.
+every iteration (by a copy kernel with streaming stores: nothing of the copy
+stays in the caches, neither inputs for the step to find nor modified lines
+for it to push out); each step is timed with HIP events on the executor's
+stream, as the reference times each iteration.
 
 value     = bytes that reach memory per step / mean step time: an HBM rate,
             at most the 8 TB/s peak.  The bytes are the plan's of this very
@@ -197,7 +199,8 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     CPU checker loaded, every element of every rank equals the checker's (null when a check was not made)."""
     import numpy as np
     from oracle import parse_table
-    out = {"legend": "ms: mean step; GBps, frac: bytes that reach memory / ms, of 8 TB/s; ok: ranks identical and every element = CPU checker"}
+    out = {"legend": "ms: mean step; GBps, frac: bytes that reach memory / ms, of 8 TB/s; ok: ranks identical and every element = CPU checker; "
+                     "placed: 1 = ranks in two regions of HBM, else -(SAR_SPREAD_* reason)"}
 
     def table(n):
         path = os.path.join(ROOT, "stragglar_amd", "schedules", "stragglar_n%d.txt" % n)
@@ -211,6 +214,11 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
         for r in range(n):
             fill(r)
         ctx.snapshot()
+
+    def placed():
+        """1 = the rank buffers lie in two regions of HBM; else the SAR_SPREAD_* reason why not, negated."""
+        st = ctx.stats()
+        return 1 if st.arena_spread else -int(st.spread_reason)
 
     def steps_ms(delay, k, w):
         for _ in range(w):
@@ -259,7 +267,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
     leg.update({"what": "pre-work + 7 rounds, %d B per rank" % nbytes,
-                "launches": 1 if st.fused_prework else int(st.launches), "ok": ok("stragglar", rounds6, "f16", 0.0, n, n - 1)})
+                "launches": 1 if st.fused_prework else int(st.launches), "placed": placed(), "ok": ok("stragglar", rounds6, "f16", 0.0, n, n - 1)})
     out["config3_n6_64MiB_f16_prework"] = leg
 
     # configs[4]: message sizes for n = 8 fp32, four algorithms, eager launches
@@ -278,6 +286,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
             st = ctx.stats()
             r = leg_rates(st, statistics.fmean(steps_ms(-1.0, k, w)))
             row[alg] = [round(r["ms"] * 1e3, 2), r["GBps"], r["frac"], ok(alg, rounds8 if alg == "stragglar" else None, "f32", -1.0, n, sched.parts)]
+        row["placed"] = placed()
         sweep[label] = row
     out["config4_sizes_n8_f32"] = sweep
 
@@ -293,7 +302,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     total = statistics.fmean(ts)
     leg = {"what": "%d B per rank, DELAY %.0f ms, pre-work beside the straggler's sleep" % (nbytes, delay),
            "ms": round(total, 5), "ms_after_arrival": round(total - delay, 5),
-           "reference_style_GiBps": round(nbytes / 2.0 ** 30 * 1000.0 / (total - delay), 2),
+           "reference_style_GiBps": round(nbytes / 2.0 ** 30 * 1000.0 / (total - delay), 2), "placed": placed(),
            "ok": ok("stragglar", rounds8, "bf16", delay, n, n - 1)}
     # the two kernels of that run, each on its own: bytes that reach memory / time of the launch
     ctx.prepare(main8, None)

@@ -316,7 +316,10 @@ int sar_fill_uniform(sar_ctx* ctx, int rank, uint64_t seed, double lo, double hi
 int sar_fill_normal(sar_ctx* ctx, int rank, uint64_t seed, double mean, double std);
 
 /* Keep / bring back a device-side copy of all rank buffers (the reference
- * re-fills before every iteration, allreduce_8GPU.cu:1009-1026). */
+ * re-fills before every iteration, allreduce_8GPU.cu:1009-1026).  sar_restore
+ * copies with streaming stores, as the fills store: a run that follows starts
+ * with nothing of its inputs in the caches and no modified lines of the copy
+ * in the Infinity Cache to push out. */
 int sar_snapshot(sar_ctx* ctx);
 int sar_restore(sar_ctx* ctx);
 
@@ -398,16 +401,17 @@ int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64
  * arena_spread), as functions of the region probe's times alone -- no device is touched; tests feed them recorded
  * times.  No counterpart in the reference (one buffer per GPU: allreduce_8GPU.cu:977-990).
  * sar_spread_yardstick: neighbours_ms = the probe's time for three pairs of neighbouring windows of the first
- * allocation, ends_ms = for its first and last window.  *yardstick_ms = the fastest of the four, the time of a pair
- * that shares a region.  Returns 0, or 1 when the ends are so much faster than the median neighbouring pair that a
- * region boundary must run through the allocation (the search then sets it aside and starts from the next one).
+ * allocation, ends_ms = for its first and last window.  *yardstick_ms = ends_ms, the time of two distant windows that
+ * share a region (or the median neighbouring pair, should that be faster).  Returns 0, or 1 when the ends are so much
+ * faster than the median neighbouring pair that a region boundary must run through the allocation (the search then
+ * sets it aside and starts from the next one).
  * sar_spread_is_elsewhere: 1 when a candidate's probe time against the first allocation says "another region"
  * (clearly below the yardstick), else 0.  Negative = SAR_EINVAL. */
 int sar_spread_yardstick(const float* neighbours_ms, float ends_ms, float* yardstick_ms);
 int sar_spread_is_elsewhere(float yardstick_ms, float probe_ms);
 /* The verdict on a whole search: probe_ms[0..n) are the candidates' times against the first allocation.  Returns 1 and
- * *pick = the candidate to take when the times fall into two populations with a clear gap -- candidates elsewhere,
- * clearly below the yardstick, and the rest at the yardstick and above, nothing in between --, else 0 and *pick = -1:
+ * *pick = the candidate to take (the fastest) when the times fall into two populations -- candidates elsewhere, clearly
+ * below the yardstick, and the rest, with a clear gap between the two in the candidates' own times --, else 0 and *pick = -1:
  * the ranks then sit in one ordinary allocation (SAR_SPREAD_NO_PAIR).  Times <= 0 are failed probes and say nothing. */
 int sar_spread_pick(float yardstick_ms, const float* probe_ms, int n, int* pick);
 

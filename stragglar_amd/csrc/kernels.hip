@@ -755,8 +755,10 @@ __device__ __forceinline__ uint16_t narrow16(float f, int dtype) {
 // fill_pattern, allreduce_8GPU.cu:41-45
 __global__ void fill_const_kernel(char* dst, uint64_t elems, float value, int dtype) {
     uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
-    if (dtype == SAR_F32) { float* d = reinterpret_cast<float*>(dst); for (; i < elems; i += stride) d[i] = value; }
-    else { uint16_t h = narrow16(value, dtype); uint16_t* d = reinterpret_cast<uint16_t*>(dst); for (; i < elems; i += stride) d[i] = h; }
+    // (streaming stores, here and in fill_random_kernel: a fill in front of a timed run must not leave a cache's worth
+    // of modified lines in the Infinity Cache for that run to push out)
+    if (dtype == SAR_F32) { float* d = reinterpret_cast<float*>(dst); for (; i < elems; i += stride) __builtin_nontemporal_store(value, d + i); }
+    else { uint16_t h = narrow16(value, dtype); uint16_t* d = reinterpret_cast<uint16_t*>(dst); for (; i < elems; i += stride) __builtin_nontemporal_store(h, d + i); }
 }
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
@@ -779,8 +781,8 @@ __global__ void fill_random_kernel(char* dst, uint64_t elems, uint64_t key, doub
             v = a + b * (((double)sum - 6.0 * 0x1p24) * 0x1p-24);
         }
         float f = (float)v;
-        if (dtype == SAR_F32) reinterpret_cast<float*>(dst)[i] = f;
-        else reinterpret_cast<uint16_t*>(dst)[i] = narrow16(f, dtype);
+        if (dtype == SAR_F32) __builtin_nontemporal_store(f, reinterpret_cast<float*>(dst) + i);
+        else __builtin_nontemporal_store(narrow16(f, dtype), reinterpret_cast<uint16_t*>(dst) + i);
     }
 }
 
@@ -792,6 +794,16 @@ __global__ void compare_kernel(const char* a, const char* b, uint64_t bytes, int
     bool bad = false;
     for (uint64_t n = bytes >> 1; i < n; i += stride) bad |= (x[i] != y[i]);
     if (bad) atomicOr(differs, 1);
+}
+
+// dst <- src, 16 bytes per lane with streaming loads and stores (the < 16 bytes behind the last whole vector byte by
+// byte): the copy that puts the inputs back before a timed run.  Streaming stores do not allocate in the 256 MB
+// Infinity Cache, so the copy leaves no modified lines there for the run that follows to push out, and no part of
+// the inputs in the caches either: the run starts cold.  Both pointers 16-byte aligned.
+__global__ __launch_bounds__(256) void copy_kernel(char* __restrict__ dst, const char* __restrict__ src, uint64_t bytes) {
+    const uint64_t nvec = bytes >> 4, step = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += step) st16<true>(dst + (i << 4), ld16<true>(src + (i << 4)));
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t)(bytes & 15u)) dst[(nvec << 4) + threadIdx.x] = src[(nvec << 4) + threadIdx.x];
 }
 
 // gpu_sleep_kernel, allreduce_8GPU.cu:36-39: one lane spins until `ticks` of
@@ -812,6 +824,15 @@ hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_
     if (elems == 0) return hipSuccess;
     uint64_t blocks = (elems + 255) / 256; if (blocks > 16384) blocks = 16384;
     hipLaunchKernelGGL(fill_random_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, dst, elems, key, a, b, mode, dtype);
+    return hipGetLastError();
+}
+hipError_t launch_copy(hipStream_t st, char* dst, const char* src, uint64_t bytes) {
+    if (bytes == 0) return hipSuccess;
+    if ((((uintptr_t)dst | (uintptr_t)src) & 15u) != 0) return hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, st);
+    uint64_t blocks = ((bytes >> 4) + 255) / 256;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(copy_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, dst, src, bytes);
     return hipGetLastError();
 }
 hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t bytes, int* differs) {

@@ -86,6 +86,8 @@ hipError_t launch_column(int dtype, int block, uint32_t grid, uint32_t nslots, h
 
 hipError_t launch_fill_const(hipStream_t st, char* dst, uint64_t elems, float value, int dtype);
 hipError_t launch_fill_random(hipStream_t st, char* dst, uint64_t elems, uint64_t key, double a, double b, int mode, int dtype);
+// device-to-device copy with streaming accesses (hipMemcpyAsync when a pointer is not 16-byte aligned)
+hipError_t launch_copy(hipStream_t st, char* dst, const char* src, uint64_t bytes);
 hipError_t launch_compare(hipStream_t st, const char* a, const char* b, uint64_t bytes, int* differs);
 // writes 4 * stream_bytes to each of the two windows; stamps[0] / stamps[1] (preset to ~0 / 0) receive the wall-clock
 // ticks of the earliest start and the latest end

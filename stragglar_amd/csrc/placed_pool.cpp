@@ -20,11 +20,16 @@ constexpr uint64_t kMinHalf = 4ull << 30;              // per allocation: eight 
 constexpr uint64_t kMaxHalf = 32ull << 30;
 constexpr uint64_t kSearch = 96ull << 30;              // candidates held while looking, beyond the pair itself: one region
 constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 streams of this size (beyond what the Infinity Cache absorbs)
-// A pair in different regions takes at most kFaster of the fastest pair within one (measured 0.85 to 0.895 on an empty
-// device, up to 0.932 with 80 GiB of other allocations around; candidates in the same region 0.98 and more), and
-// nothing may lie within kGap above the slowest candidate that counts as elsewhere: the two populations must not
-// run into each other.
-constexpr float kFaster = 0.95f, kGap = 0.03f;
+// What separates the two populations of probe times.  Two windows that share a region take 181-228 us and scatter (which
+// banks collide is a matter of the exact addresses); two windows in different regions take 158-167 us whatever the
+// addresses.  The yardstick is the probe's time for the two ENDS of the first allocation (181-189 us in every search on
+// record), or the median of its three neighbouring pairs should that be faster.  The fastest of all four was tried first
+// and drifts: in an allocation pieced together from freed memory one neighbouring pair read 173-175 us, which pulled
+// candidates elsewhere at 162-167 us above the limit.  Against the yardstick candidates elsewhere come in at 0.85-0.90
+// on an empty device and 0.932 with 80 GiB of other allocations around, candidates of the same region at 0.98 and more.
+// The candidates' own times must show the gap as well: at least kGap between the slowest "elsewhere" and the fastest
+// other candidate (measured 11-18 %).
+constexpr float kFaster = 0.95f, kGap = 0.04f;
 constexpr float kStraddle = 0.86f;                     // the two ends of an allocation against its neighbouring windows: below this a
                                                        // boundary runs through it (measured 0.80 with a boundary, 0.90 to 0.93 without)
 
@@ -120,11 +125,11 @@ void free_pair(Pool& p) {
 // Candidates are allocated one after the other (nothing is assumed about the order in which the driver hands out
 // memory) and each is timed against the first with a short probe: eight write streams of 128 MiB, four in either
 // allocation.  The yardstick is the probe's own time for windows that do share a region, not a fixed figure: the
-// fastest of four pairs of windows of the first allocation (measured 181-213 us; candidates in the same region
-// 183-217 us, elsewhere 158-165 us).  ALL candidates within the budget are probed -- enough of them to cross a region
+// two ends of the first allocation against each other (measured 181-189 us; candidates in the same region 183-228 us,
+// elsewhere 158-167 us).  ALL candidates within the budget are probed -- enough of them to cross a region
 // boundary from anywhere, one region's worth -- and the verdict is taken on the whole set (spread_pick): the times must
-// fall into two populations with a clear gap, and the candidate taken must confirm its time on other windows of both
-// allocations.  Everything else is given back.  A wrong verdict would cost speed, not correctness; without a clear
+// fall into two populations with a clear gap, one of them clearly below the yardstick, and the candidate taken must
+// confirm its time on other windows of both allocations.  Everything else is given back.  A wrong verdict would cost speed, not correctness; without a clear
 // one the caller's ranks sit in an ordinary allocation.
 int find_pair(const ProbeEnv& env, uint64_t half, Pool& p) {
     const uint64_t window = 4 * kProbeStream;
@@ -257,7 +262,7 @@ bool valid(int device) { return device >= 0 && device < kMaxDevices; }
 bool spread_yardstick(const float neighbours_ms[3], float ends_ms, float* yardstick_ms) {
     float adj[3] = {neighbours_ms[0], neighbours_ms[1], neighbours_ms[2]};
     std::sort(adj, adj + 3);
-    *yardstick_ms = std::min(ends_ms, adj[0]);
+    *yardstick_ms = std::min(ends_ms, adj[1]);
     return !(ends_ms < kStraddle * adj[1]);
 }
 
@@ -265,19 +270,23 @@ bool spread_is_elsewhere(float yardstick_ms, float probe_ms_value) { return prob
 
 int spread_pick(float yardstick_ms, const float* t, int n) {
     if (!(yardstick_ms > 0.f) || !t || n < 1) return -1;
+    // the candidates clearly below the yardstick, and the fastest of the rest
     int best = -1;
-    float slowest_elsewhere = 0.f, fastest_other = yardstick_ms;      // the yardstick itself is a time within one region
+    float slowest_elsewhere = 0.f, fastest_other = 0.f;
     for (int i = 0; i < n; ++i) {
         if (!(t[i] > 0.f)) continue;                                  // a failed probe says nothing
         if (spread_is_elsewhere(yardstick_ms, t[i])) {
             slowest_elsewhere = std::max(slowest_elsewhere, t[i]);
             if (best < 0 || t[i] < t[best]) best = i;
-        } else {
-            fastest_other = std::min(fastest_other, t[i]);
+        } else if (fastest_other == 0.f || t[i] < fastest_other) {
+            fastest_other = t[i];
         }
     }
     if (best < 0) return -1;
-    return fastest_other - slowest_elsewhere >= kGap * yardstick_ms ? best : -1;
+    // ... and the gap between the two populations, in the candidates' own times (every candidate elsewhere: nothing to compare with,
+    // the yardstick has spoken)
+    if (fastest_other > 0.f && fastest_other < (1.f + kGap) * slowest_elsewhere) return -1;
+    return best;
 }
 
 void pool_attach(int device, const void* owner) {

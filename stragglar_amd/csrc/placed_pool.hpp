@@ -27,15 +27,15 @@ struct SearchRecord {
 };
 
 // ---- the decisions of the search, as functions of probe times alone (checked against recorded times without a device)
-// Yardstick: the fastest of four pairs of windows within the first allocation (three neighbouring pairs and its two
-// ends).  False when the ends probe so much faster than the median neighbouring pair that a region boundary must
-// run through the allocation.
+// Yardstick: the probe's time for the two ends of the first allocation (or the median of three neighbouring pairs of
+// its windows, should that be faster).  False when the ends probe so much faster than the median neighbouring pair
+// that a region boundary must run through the allocation.
 bool spread_yardstick(const float neighbours_ms[3], float ends_ms, float* yardstick_ms);
 // A single probe against the first allocation says "another region": clearly below the yardstick.
 bool spread_is_elsewhere(float yardstick_ms, float probe_ms);
-// All candidates' probe times at once: the index of the candidate to take when the times fall into two populations
-// with a clear gap between them (candidates elsewhere, clearly below the yardstick; candidates in the same region,
-// at the yardstick and above), else -1: nobody is clearly elsewhere, or the populations run into each other.
+// All candidates' probe times at once: the index of the candidate to take (the fastest) when the times fall into two
+// populations -- candidates elsewhere, clearly below the yardstick, and the rest, with a clear gap between the two in
+// the candidates' own times --, else -1: nobody is clearly elsewhere, or the populations run into each other.
 int spread_pick(float yardstick_ms, const float* probe_ms, int n);
 
 // ---- the pool ------------------------------------------------------------------------------------------------

@@ -277,8 +277,8 @@ def test_bench_default_workload_carries_every_baseline_config():
     assert c3["ok"] is True and c3["launches"] == 1 and abs(c3["memory_bytes"] - 12 * 67112960) <= 67112960 // 100
     sweep = other["config4_sizes_n8_f32"]
     for size in ("4KiB", "64KiB", "1MiB", "16MiB", "256MiB", "1GiB"):
-        assert sorted(sweep[size]) == ["direct", "rhd", "ring", "stragglar"]
-        for us, gbps, frac, ok in sweep[size].values():
+        assert sorted(sweep[size]) == ["direct", "placed", "rhd", "ring", "stragglar"]
+        for us, gbps, frac, ok in (sweep[size][a] for a in ("stragglar", "ring", "rhd", "direct")):
             assert us > 0 and gbps > 0 and ok is True
     assert sweep["1GiB"]["stragglar"][2] > 0.5                                                  # an HBM rate at this size
     c2 = other["config2_n8_1GiB_bf16_delay5ms"]

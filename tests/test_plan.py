@@ -503,9 +503,8 @@ def test_rows_that_share_a_cell_do_not_take_their_operands_together(sarlib):
     assert any(r.joins for r in second)
 
 
-# Region probe times recorded on MI355X boxes (microseconds): per search the three neighbouring pairs of windows of the
-# first allocation, its two ends, the times of candidates that share its region and of the pair that lay elsewhere
-# (first probe, second probe on other windows).
+# Probe times (us) of recorded searches on MI355X: the three neighbouring pairs of windows within the first allocation,
+# its two ends, the times of candidates that share its region and of candidates that lay elsewhere.
 _RECORDED_SEARCHES = [
     ((180.8, 205.7, 198.9), 185.2, (185.5, 190.4, 212.0, 197.7, 201.3), (160.4, 158.5)),
     ((202.0, 204.5, 200.1), 181.5, (182.8, 184.9, 190.0, 195.1), (158.3, 159.3)),
@@ -514,48 +513,55 @@ _RECORDED_SEARCHES = [
     ((192.7, 194.5, 209.1), 184.5, (216.9, 187.2), (161.0, 163.5)),
     ((200.8, 202.1, 202.2), 189.1, (193.3,), (165.4, 163.8)),
     ((198.0, 200.2, 202.1), 186.9, (), (162.8, 162.8)),
+    # a fresh process, 4 GiB candidates: 22 in the region of the first allocation before the first one elsewhere
+    ((188.0, 200.7, 197.3), 185.8, (186.8, 193.0, 185.1, 191.3, 213.4, 220.0, 199.5, 200.4, 193.6, 191.9, 189.4, 193.7, 215.8, 225.5, 201.9,
+                                   203.6, 191.7, 191.8, 186.6, 187.4, 212.5, 228.5), (159.1, 160.2, 159.1)),
+    # the pair looked for again in memory that earlier allocations had cut up: one pair of windows WITHIN the first
+    # allocation reads 175 / 174 us, and candidates elsewhere come first, in between and last
+    ((175.2, 209.9, 202.9), 186.0, (211.5, 193.2, 194.0, 206.3, 215.6, 192.9), (163.0, 162.2, 164.0, 163.1, 162.1, 161.9, 162.5, 166.5)),
+    ((173.6, 204.0, 217.6), 185.7, (197.9, 191.1, 217.6, 188.3, 193.3, 209.8, 203.4, 188.0), (160.4, 161.2, 166.7, 162.4, 164.4)),
 ]
 
 
 def test_region_search_decisions_on_recorded_probe_times(sarlib):
-    """The yardstick is the fastest pair of windows within the first allocation; a candidate lies elsewhere only when it is
-    clearly faster than that.  An earlier form compared against ONE neighbouring pair (up to 213 us) and took candidates of
-    the same region at 183-190 us for another region: those must be turned down, and an allocation whose ends are merely
-    the fastest of its own pairs must not be mistaken for one with a boundary in it."""
+    """The yardstick is the probe's time for the two ends of the first allocation (the median neighbouring pair if
+    that is faster); a candidate lies elsewhere only when it is clearly faster than that AND the candidates' own times
+    show two populations with a gap.  Earlier forms failed both ways on these records: a yardstick from ONE neighbouring
+    pair (up to 213 us) took candidates of the same region at 183-190 us for another region; the fastest of all four
+    pairs as the yardstick (173-175 us in memory that had been cut up) turned down candidates elsewhere at 162-167 us."""
+    import statistics
     for neighbours, ends, same_region, elsewhere in _RECORDED_SEARCHES:
         y, straddles = sarlib.spread_yardstick([t * 1e-3 for t in neighbours], ends * 1e-3)
         assert not straddles, (neighbours, ends)
-        assert abs(y * 1e3 - min(min(neighbours), ends)) < 1e-3
+        assert abs(y * 1e3 - min(ends, statistics.median(neighbours))) < 1e-3
         for t in same_region:
             assert not sarlib.spread_is_elsewhere(y, t * 1e-3), (neighbours, ends, t)
         for t in elsewhere:
             assert sarlib.spread_is_elsewhere(y, t * 1e-3), (neighbours, ends, t)
+        # the verdict on the whole search, candidates in any order: the fastest candidate elsewhere
+        times = [t * 1e-3 for t in same_region] + [t * 1e-3 for t in elsewhere]
+        want = len(same_region) + min(range(len(elsewhere)), key=lambda k: elsewhere[k])
+        assert sarlib.spread_pick(y, times) == want, (neighbours, ends)
+        assert sarlib.spread_pick(y, times[::-1]) == len(times) - 1 - max(k for k in range(len(times)) if times[k] == times[want]), (neighbours, ends)
+        assert sarlib.spread_pick(y, [t * 1e-3 for t in same_region]) == -1          # nobody elsewhere: no pair
+    # the search with 80 GiB of other allocations around: the fastest pair within the first allocation at 174-175 us,
+    # the pair that was kept at 163 us (0.932 of that; about 0.90 of a median around 181 us)
+    y, _ = sarlib.spread_yardstick([0.1800, 0.1830, 0.1880], 0.1745)
+    assert sarlib.spread_pick(y, [0.1761, 0.1790, 0.1810, 0.1627]) == 3
+    # two populations that run into each other: a candidate under the limit with another right above it is not a clear verdict
+    assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1776]) == -1
+    assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1813]) == 1
+    assert sarlib.spread_pick(0.185, [0.1700]) == 0                                   # every candidate elsewhere: the yardstick has spoken
+    assert sarlib.spread_pick(0.185, [0.1770]) == -1                                  # 0.957: not below the limit
+    # failed probes say nothing, and no candidates is no pair
+    assert sarlib.spread_pick(0.185, [-1.0, 0.0, 0.158]) == 2
+    assert sarlib.spread_pick(0.185, [-1.0]) == -1
+    assert sarlib.spread_pick(0.185, []) == -1
     # a boundary inside the first allocation: its ends probe like a pair in two regions, its neighbouring windows do not
     y, straddles = sarlib.spread_yardstick([0.199, 0.203, 0.160], 0.159)
     assert straddles
     # ... and with such a yardstick nothing would pass, so the search sets the allocation aside instead of using it
     assert not sarlib.spread_is_elsewhere(y, 0.159)
-    # The verdict on a whole search: the candidates' times must fall into two populations with a clear gap.
-    for neighbours, ends, same_region, elsewhere in _RECORDED_SEARCHES:
-        y, _ = sarlib.spread_yardstick([t * 1e-3 for t in neighbours], ends * 1e-3)
-        times = [t * 1e-3 for t in same_region] + [elsewhere[0] * 1e-3]
-        assert sarlib.spread_pick(y, times) == len(times) - 1, (neighbours, ends)
-        assert sarlib.spread_pick(y, [t * 1e-3 for t in same_region]) == -1          # nobody elsewhere: no pair
-    # the search with 80 GiB of other allocations around: the yardstick drops to 174-175 us and the pair comes in at
-    # 0.932 of it, candidates in the same region at 0.98 and more: still two populations
-    assert sarlib.spread_pick(0.1745, [0.1761, 0.1718, 0.1810, 0.1627]) == 3
-    # two candidates elsewhere (the other two regions): the faster one
-    assert sarlib.spread_pick(0.185, [0.190, 0.160, 0.186, 0.158]) == 3
-    # populations that run into each other: a candidate at 0.94 of the yardstick with another at 0.96 right above it
-    # is not a clear verdict (the same candidate with the next one at 0.98 is)
-    assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1776]) == -1
-    assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1813]) == 1
-    assert sarlib.spread_pick(0.170, [0.1560]) == 0                                   # 0.918, alone: clear of the yardstick itself
-    assert sarlib.spread_pick(0.170, [0.1620]) == -1                                  # 0.953: not below the limit
-    # failed probes say nothing, and no candidates is no pair
-    assert sarlib.spread_pick(0.185, [-1.0, 0.0, 0.158]) == 2
-    assert sarlib.spread_pick(0.185, [-1.0]) == -1
-    assert sarlib.spread_pick(0.185, []) == -1
     # failed probes (negative) and nonsense never count as elsewhere; bad arguments are refused
     assert not sarlib.spread_is_elsewhere(0.185, -1.0)
     assert not sarlib.spread_is_elsewhere(0.185, 0.0)
