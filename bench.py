@@ -489,13 +489,13 @@ def main():
 
     if args.alg == "stragglar" and st.col_slots and 2 <= n - 1 <= 8:
         # What the memory system delivers for this kernel's own mix of streams, by a kernel that does nothing else
-        # (sar_probe_streams, fastest of 72 launch shapes): per chunk index r the cold reads of rank r's and the
+        # (sar_probe_streams, fastest of 108 launch shapes): per chunk index r the cold reads of rank r's and the
         # straggler's chunk r and the stores of their sum to every rank, on the same buffers in the same places.
         chunk = (elems // (n - 1)) * 4
         res = ctx.probe_streams([([r, n - 1], list(range(n)), r * chunk) for r in range(n - 1)], chunk - chunk % 16, 5)
         rec["stream_ceiling"] = {"mix": "%d x (2 streams read + %d written), %d B each: the schedule's traffic once re-reads come from LDS" % (n - 1, n, chunk - chunk % 16),
                                  "GBps": round(res.gbps, 1), "frac_of_hbm_peak": round(res.gbps / HBM_PEAK_GBPS, 4), "ms": round(res.best_ms, 5),
-                                 "shape": {"block": res.block, "vectors_per_thread": res.unroll, "streaming": res.nontemporal, "resident_grid": res.persistent, "jobs_take_turns": res.interleave},
+                                 "shape": {"block": res.block, "vectors_per_thread": res.unroll, "cache_mode": res.nontemporal, "resident_grid": res.persistent, "jobs_take_turns": res.interleave},
                                  "shapes_tried": res.variants, "slowest_shape_ms": round(res.worst_ms, 5),
                                  "kernel_vs_ceiling": round(roofline["achieved"] / res.gbps, 4)}
         ctx.restore()

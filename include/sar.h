@@ -377,8 +377,8 @@ int sar_launch_bytes(sar_ctx* ctx, uint64_t* bytes, int cap, int* count);
  * is nread streams read and nwrite streams written, each `bytes` long, starting byte_off into the named ranks'
  * buffers; every 16-byte vector written is the fp32 sum of the job's read streams.  A rank named on both sides is
  * updated in place, as the two sides of an exchange are (allreduce_8GPU.cu:564-578 followed by reduce_add :29-34).
- * All jobs of a call run in one launch of a kernel that does nothing else, in 36 (one job) or 72 shapes --
- * 256/512/1024 threads x 1/2/4 vectors per thread x cached/streaming accesses x one tile per workgroup or a
+ * All jobs of a call run in one launch of a kernel that does nothing else, in 54 (one job) or 108 shapes --
+ * 256/512/1024 threads x 1/2/4 vectors per thread x cached / streaming loads with cached stores / streaming loads and stores x one tile per workgroup or a
  * resident grid x jobs one after the other or taking turns --, each timed `reps` times with events after one
  * warm-up launch; the result names the fastest shape.  THE RANK BUFFERS ARE OVERWRITTEN. */
 typedef struct sar_probe_job {
@@ -388,11 +388,12 @@ typedef struct sar_probe_job {
 } sar_probe_job;
 typedef struct sar_probe_result {
     float best_ms, worst_ms;          /* fastest and slowest shape (each the minimum over its reps) */
-    int32_t block, unroll, nontemporal, persistent, interleave;      /* the fastest shape */
+    int32_t block, unroll, nontemporal, persistent, interleave;      /* the fastest shape; nontemporal: 0 = cached accesses, */
+                                      /* 1 = streaming loads and cached stores, 2 = streaming loads and stores */
     int32_t variants;                 /* shapes tried */
     uint64_t bytes_moved;             /* (nread + nwrite) * bytes summed over the jobs */
-    float variant_ms[72];             /* every shape's time, in the order they are tried: threads 256, 512, 1024 (slowest     */
-                                      /* index) x vectors 1, 2, 4 x cached, streaming x tile per workgroup, resident grid x   */
+    float variant_ms[108];            /* every shape's time, in the order they are tried: threads 256, 512, 1024 (slowest     */
+                                      /* index) x vectors 1, 2, 4 x the three cache modes x tile per workgroup, resident grid x */
                                       /* jobs one after the other, taking turns (fastest index; one job: this level is absent) */
 } sar_probe_result;
 int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64_t bytes, int reps, sar_probe_result* out);

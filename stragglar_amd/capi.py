@@ -71,15 +71,16 @@ class ProbeJob(ctypes.Structure):
 class ProbeResult(ctypes.Structure):
     _fields_ = [("best_ms", ctypes.c_float), ("worst_ms", ctypes.c_float), ("block", ctypes.c_int32), ("unroll", ctypes.c_int32),
                 ("nontemporal", ctypes.c_int32), ("persistent", ctypes.c_int32), ("interleave", ctypes.c_int32),
-                ("variants", ctypes.c_int32), ("bytes_moved", ctypes.c_uint64), ("variant_ms", ctypes.c_float * 72)]
+                ("variants", ctypes.c_int32), ("bytes_moved", ctypes.c_uint64), ("variant_ms", ctypes.c_float * 108)]
 
     def shapes(self):
-        """(block, vectors per thread, streaming, resident grid, jobs take turns, ms) of every shape tried."""
+        """(block, vectors per thread, cache mode, resident grid, jobs take turns, ms) of every shape tried; cache mode
+        0 = cached accesses, 1 = streaming loads and cached stores, 2 = streaming loads and stores."""
         out, k = [], 0
-        turns = (0, 1) if self.variants == 72 else (0,)
+        turns = (0, 1) if self.variants == 108 else (0,)
         for block in (256, 512, 1024):
             for unroll in (1, 2, 4):
-                for nt in (0, 1):
+                for nt in (0, 1, 2):
                     for persistent in (0, 1):
                         for il in turns:
                             out.append((block, unroll, nt, persistent, il, self.variant_ms[k]))

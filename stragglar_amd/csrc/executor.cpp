@@ -1225,20 +1225,20 @@ static int probe_streams_body(sar_ctx* c, int njobs, const sar_probe_job* jobs, 
     out->bytes_moved = moved;
     for (int block : {256, 512, 1024})
         for (int unroll : {1, 2, 4})
-            for (int nt = 0; nt < 2; ++nt)
+            for (int nt = 0; nt < 3; ++nt)
                 for (int persistent = 0; persistent < 2; ++persistent)
                     for (int interleave = 0; interleave < (njobs > 1 ? 2 : 1); ++interleave) {
                         float best = -1.f;
                         for (int r = 0; r <= reps; ++r) {                   // the first run warms up and is not counted
                             SAR_HIP(hipEventRecord(c->ev_prof[0], c->stream));
-                            SAR_HIP(sar::launch_stream_probe(c->stream, J, block, unroll, nt != 0, persistent != 0, interleave != 0, c->cu_count));
+                            SAR_HIP(sar::launch_stream_probe(c->stream, J, block, unroll, nt, persistent != 0, interleave != 0, c->cu_count));
                             SAR_HIP(hipEventRecord(c->ev_prof[1], c->stream));
                             SAR_HIP(hipEventSynchronize(c->ev_prof[1]));
                             float ms = 0.f;
                             SAR_HIP(hipEventElapsedTime(&ms, c->ev_prof[0], c->ev_prof[1]));
                             if (r > 0 && (best < 0.f || ms < best)) best = ms;
                         }
-                        if (out->variants < 72) out->variant_ms[out->variants] = best;
+                        if (out->variants < 108) out->variant_ms[out->variants] = best;
                         out->variants += 1;
                         if (out->best_ms <= 0.f || best < out->best_ms) {
                             out->best_ms = best; out->block = block; out->unroll = unroll; out->nontemporal = nt;

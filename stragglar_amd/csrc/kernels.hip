@@ -870,9 +870,11 @@ hipError_t launch_region_probe(hipStream_t st, char* a, char* b, uint64_t stream
 // of a job is the fp32 sum of its read streams (a constant when there is none), stored to each of its written
 // streams.  A stream that is both read and written is updated in place, as an exchange does.  Tiles of BLOCK * U
 // vectors, one per workgroup (PERSIST = false: the dispatcher hands them out) or a grid of 8 workgroups per CU
-// striding over them; tiles job by job or, `interleave`, the jobs taking turns.
-template <int R, int U, bool NT, bool PERSIST>
+// striding over them; tiles job by job or, `interleave`, the jobs taking turns.  POL as for the column kernel: 0 = cached
+// accesses, 1 = streaming loads and cached stores, 2 = streaming loads and stores.
+template <int R, int U, int POL, bool PERSIST>
 __global__ __launch_bounds__(1024) void stream_probe_kernel(ProbeJobs J, uint32_t tiles_per_job, uint32_t interleave) {
+    constexpr bool LNT = POL >= 1, SNT = POL == 2;
     const uint32_t ntiles = tiles_per_job * J.njobs;
     const uint64_t nvec = J.bytes >> 4;
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += PERSIST ? gridDim.x : ntiles) {
@@ -888,42 +890,42 @@ __global__ __launch_bounds__(1024) void stream_probe_kernel(ProbeJobs J, uint32_
             v[u] = R ? f4{0.f, 0.f, 0.f, 0.f} : f4{1.f, 2.f, 3.f, 4.f};
             if (whole || i < nvec) {
 #pragma unroll
-                for (int k = 0; k < R; ++k) v[u] += ld16<NT>(J.rd[job][k] + (i << 4));
+                for (int k = 0; k < R; ++k) v[u] += ld16<LNT>(J.rd[job][k] + (i << 4));
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint64_t i = first + (uint64_t)u * blockDim.x;
             if (whole || i < nvec)
-                for (uint32_t w = 0; w < nw; ++w) st16<NT>(J.wr[job][w] + (i << 4), v[u]);
+                for (uint32_t w = 0; w < nw; ++w) st16<SNT>(J.wr[job][w] + (i << 4), v[u]);
         }
     }
 }
 
 template <int R>
-static hipError_t launch_stream_probe_r(hipStream_t st, const ProbeJobs& J, uint32_t grid, int block, uint32_t tiles_per_job, int unroll, bool nontemporal, bool persistent, uint32_t il) {
-#define SAR_PROBE(U, NT, P) hipLaunchKernelGGL((stream_probe_kernel<R, U, NT, P>), dim3(grid), dim3(block), 0, st, J, tiles_per_job, il)
-    switch (unroll * 4 + (nontemporal ? 2 : 0) + (persistent ? 1 : 0)) {
-        case 1 * 4 + 0: SAR_PROBE(1, false, false); break;
-        case 1 * 4 + 1: SAR_PROBE(1, false, true); break;
-        case 1 * 4 + 2: SAR_PROBE(1, true, false); break;
-        case 1 * 4 + 3: SAR_PROBE(1, true, true); break;
-        case 2 * 4 + 0: SAR_PROBE(2, false, false); break;
-        case 2 * 4 + 1: SAR_PROBE(2, false, true); break;
-        case 2 * 4 + 2: SAR_PROBE(2, true, false); break;
-        case 2 * 4 + 3: SAR_PROBE(2, true, true); break;
-        case 4 * 4 + 0: SAR_PROBE(4, false, false); break;
-        case 4 * 4 + 1: SAR_PROBE(4, false, true); break;
-        case 4 * 4 + 2: SAR_PROBE(4, true, false); break;
-        case 4 * 4 + 3: SAR_PROBE(4, true, true); break;
+static hipError_t launch_stream_probe_r(hipStream_t st, const ProbeJobs& J, uint32_t grid, int block, uint32_t tiles_per_job, int unroll, int policy, bool persistent, uint32_t il) {
+#define SAR_PROBE(U, POL, P) hipLaunchKernelGGL((stream_probe_kernel<R, U, POL, P>), dim3(grid), dim3(block), 0, st, J, tiles_per_job, il)
+#define SAR_PROBE_U(U)                                                                        \
+    switch (policy * 2 + (persistent ? 1 : 0)) {                                              \
+        case 0: SAR_PROBE(U, 0, false); break; case 1: SAR_PROBE(U, 0, true); break;          \
+        case 2: SAR_PROBE(U, 1, false); break; case 3: SAR_PROBE(U, 1, true); break;          \
+        case 4: SAR_PROBE(U, 2, false); break; case 5: SAR_PROBE(U, 2, true); break;          \
+        default: return hipErrorInvalidValue;                                                 \
+    }
+    switch (unroll) {
+        case 1: SAR_PROBE_U(1) break;
+        case 2: SAR_PROBE_U(2) break;
+        case 4: SAR_PROBE_U(4) break;
         default: return hipErrorInvalidValue;
     }
+#undef SAR_PROBE_U
 #undef SAR_PROBE
     return hipGetLastError();
 }
 
 // All jobs of a launch read the same number of streams (J.nread[0]); the written streams may differ in number.
-hipError_t launch_stream_probe(hipStream_t st, const ProbeJobs& J, int block, int unroll, bool nontemporal, bool persistent, bool interleave, int compute_units) {
+hipError_t launch_stream_probe(hipStream_t st, const ProbeJobs& J, int block, int unroll, int policy, bool persistent, bool interleave, int compute_units) {
+    if (policy < 0 || policy > 2) return hipErrorInvalidValue;
     if (J.njobs == 0 || J.njobs > 8 || J.bytes < 16 || (block != 256 && block != 512 && block != 1024)) return hipErrorInvalidValue;
     for (uint32_t j = 0; j < J.njobs; ++j) if (J.nread[j] != J.nread[0] || J.nread[j] > 8 || J.nwrite[j] > 8) return hipErrorInvalidValue;
     const uint64_t tile_vecs = (uint64_t)block * (uint64_t)unroll;
@@ -933,15 +935,15 @@ hipError_t launch_stream_probe(hipStream_t st, const ProbeJobs& J, int block, in
     const uint32_t grid = persistent ? (uint32_t)std::min<uint64_t>(ntiles, (uint64_t)std::max(1, compute_units) * 8u) : ntiles;
     const uint32_t il = interleave ? 1u : 0u;
     switch (J.nread[0]) {
-        case 0: return launch_stream_probe_r<0>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 1: return launch_stream_probe_r<1>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 2: return launch_stream_probe_r<2>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 3: return launch_stream_probe_r<3>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 4: return launch_stream_probe_r<4>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 5: return launch_stream_probe_r<5>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 6: return launch_stream_probe_r<6>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        case 7: return launch_stream_probe_r<7>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
-        default: return launch_stream_probe_r<8>(st, J, grid, block, tpj, unroll, nontemporal, persistent, il);
+        case 0: return launch_stream_probe_r<0>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 1: return launch_stream_probe_r<1>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 2: return launch_stream_probe_r<2>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 3: return launch_stream_probe_r<3>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 4: return launch_stream_probe_r<4>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 5: return launch_stream_probe_r<5>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 6: return launch_stream_probe_r<6>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        case 7: return launch_stream_probe_r<7>(st, J, grid, block, tpj, unroll, policy, persistent, il);
+        default: return launch_stream_probe_r<8>(st, J, grid, block, tpj, unroll, policy, persistent, il);
     }
 }
 

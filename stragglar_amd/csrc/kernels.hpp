@@ -100,7 +100,8 @@ struct ProbeJobs {
     uint32_t njobs, reserved;
     uint64_t bytes;
 };
-hipError_t launch_stream_probe(hipStream_t st, const ProbeJobs& J, int block, int unroll, bool nontemporal, bool persistent, bool interleave, int compute_units);
+// policy: 0 = cached accesses, 1 = streaming loads and cached stores, 2 = streaming loads and stores
+hipError_t launch_stream_probe(hipStream_t st, const ProbeJobs& J, int block, int unroll, int policy, bool persistent, bool interleave, int compute_units);
 hipError_t launch_sleep(hipStream_t st, uint64_t ticks);
 
 }  // namespace sar

@@ -4,7 +4,7 @@
     python -m stragglar_amd.stream_probe [--ranks 8] [--mib 256] [--dtype f32] [--reps 5] [--spread 1]
 
 The rank buffers are allocated as for a run (padded as pad_buffers.py pads, placed by sar_alloc_ranks) and the
-library's stream probe -- a kernel that only loads, adds and stores, tried in 36 or 72 launch shapes, the fastest
+library's stream probe -- a kernel that only loads, adds and stores, tried in 54 or 108 launch shapes, the fastest
 counted -- moves the same bytes between the same addresses as
 
     exchanges   the reduce steps of the StragglAR table alone: per chunk r, rank r's and the straggler's chunk r
@@ -72,7 +72,7 @@ def main(argv=None) -> int:
     st = ctx.stats()
     print("n=%d, %d B per rank (%s), chunk %d B, rank buffers in two regions of HBM: %d (%s)"
           % (n, nbytes, args.dtype, chunk, st.arena_spread, capi.SPREAD_REASONS.get(st.spread_reason, "?")))
-    print("mix,streams,bytes_moved,us,GB/s,frac_of_8TBps,best_shape(block/vectors/streaming/resident/turns),slowest_shape_us,shapes")
+    print("mix,streams,bytes_moved,us,GB/s,frac_of_8TBps,best_shape(block/vectors/cache_mode/resident/turns),slowest_shape_us,shapes")
     want = [m for m in args.mix.split(",") if m]
     for name, jobs, size in mixes(n, chunk, nbytes - nbytes % 16, es):
         if want and name not in want:

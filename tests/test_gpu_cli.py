@@ -251,7 +251,7 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
             assert leg["ranks_identical_after_run"] is True and leg["ms_per_step"] > 0 and leg["memory_side_GBps"] > 0
             assert leg["bit_exact_vs_cpu_checker"] is True
     if "--alg" not in extra and "--forward" not in extra and "--executor" not in extra:
-        assert 0 < rec["stream_ceiling"]["GBps"] and rec["stream_ceiling"]["shapes_tried"] == 72
+        assert 0 < rec["stream_ceiling"]["GBps"] and rec["stream_ceiling"]["shapes_tried"] == 108
     if "--no-cpu" not in extra:
         base = rec["cpu_baseline"]
         assert base["kind"] == "port" and base["cores"] == 1 and base["value"] > 0 and base["unit"] == "GB/s" and base["sample"]

@@ -1004,19 +1004,19 @@ def test_stream_probe(gpu_ctx, sarlib):
     off, length = 16 * 5, 16 * 700                                       # bytes
     lo, hi = off // 4, (off + length) // 4
     res = ctx.probe_streams([([0, 1, 2], [3, 4], off), ([5, 6, 7], [5], off)], length, reps=1)
-    assert res.variants == 72 and res.best_ms > 0 and res.worst_ms >= res.best_ms and res.bytes_moved == (5 + 4) * length
+    assert res.variants == 108 and res.best_ms > 0 and res.worst_ms >= res.best_ms and res.bytes_moved == (5 + 4) * length
     assert res.block in (256, 512, 1024) and res.unroll in (1, 2, 4)
     want = inputs[0][lo:hi] + inputs[1][lo:hi] + inputs[2][lo:hi]
     for r in (3, 4):
         got = ctx.download(r)
         assert np.array_equal(got[lo:hi], want) and np.array_equal(got[:lo], inputs[r][:lo]) and np.array_equal(got[hi:], inputs[r][hi:])
-    # in place: rank 5 is read and written by every launch, 72 shapes x 2 launches each: s <- s + x6 + x7 every time
+    # in place: rank 5 is read and written by every launch, 108 shapes x 2 launches each: s <- s + x6 + x7 every time
     got = ctx.download(5)
-    assert np.array_equal(got[lo:hi], inputs[5][lo:hi] + 144 * (inputs[6][lo:hi] + inputs[7][lo:hi]))
+    assert np.array_equal(got[lo:hi], inputs[5][lo:hi] + 216 * (inputs[6][lo:hi] + inputs[7][lo:hi]))
     for r in (0, 1, 2, 6, 7):
         assert np.array_equal(ctx.download(r), inputs[r])
     res = ctx.probe_streams([([], [0, 1], 0)], 16 * 64, reps=1)
-    assert res.variants == 36
+    assert res.variants == 54
     assert np.array_equal(ctx.download(1)[:8], np.array([1, 2, 3, 4, 1, 2, 3, 4], np.float32))
     for bad in ([([0], [1], 4)],                      # not on a 16-byte boundary
                 [([0], [8], 0)],                      # no such rank
