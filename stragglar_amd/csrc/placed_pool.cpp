@@ -44,7 +44,7 @@ struct Pool {
     SearchRecord rec;
 };
 
-std::mutex g_mutex;
+std::mutex g_mutex[kMaxDevices];                      // one per GPU: a search on one does not hold up the others
 Pool g_pool[kMaxDevices];
 
 uint64_t up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
@@ -291,7 +291,7 @@ int spread_pick(float yardstick_ms, const float* t, int n) {
 
 void pool_attach(int device, const void* owner) {
     if (!valid(device)) return;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     Pool& p = g_pool[device];
     if (std::find(p.users.begin(), p.users.end(), owner) == p.users.end()) p.users.push_back(owner);
     p.rec.users = (int)p.users.size();
@@ -299,18 +299,20 @@ void pool_attach(int device, const void* owner) {
 
 void pool_detach(int device, const void* owner) {
     if (!valid(device)) return;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     Pool& p = g_pool[device];
     p.leases.erase(std::remove_if(p.leases.begin(), p.leases.end(), [&](const Lease& l) { return l.owner == owner; }), p.leases.end());
     p.users.erase(std::remove(p.users.begin(), p.users.end(), owner), p.users.end());
     p.rec.users = (int)p.users.size();
+    if (p.va && hipSetDevice(device) != hipSuccess) (void)hipGetLastError();
     if (p.users.empty() && p.va) { (void)hipDeviceSynchronize(); free_pair(p); }
     else shrink_if_idle(p);
 }
 
 int pool_lease_arena(const ProbeEnv& env, const void* owner, uint64_t lo_bytes, uint64_t hi_bytes, char** lo, char** hi) {
     if (!valid(env.device) || !lo || !hi) return SAR_SPREAD_NO_MEMORY;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[env.device]);
+    if (hipSetDevice(env.device) != hipSuccess) { (void)hipGetLastError(); return SAR_SPREAD_NO_MEMORY; }
     Pool& p = g_pool[env.device];
     release(p, owner, false);                                  // an owner holds one arena at a time
     const uint64_t lo_len = up(lo_bytes, kGranule), hi_len = up(hi_bytes, kGranule);
@@ -328,7 +330,8 @@ int pool_lease_arena(const ProbeEnv& env, const void* owner, uint64_t lo_bytes, 
 
 int pool_lease_rows(const ProbeEnv& env, const void* owner, uint64_t lo_bytes, uint64_t hi_bytes, char** base) {
     if (!valid(env.device) || !base) return SAR_SPREAD_NO_MEMORY;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[env.device]);
+    if (hipSetDevice(env.device) != hipSuccess) { (void)hipGetLastError(); return SAR_SPREAD_NO_MEMORY; }
     Pool& p = g_pool[env.device];
     release(p, owner, true);
     const int reason = ensure_pair(env, p, std::max(lo_bytes, hi_bytes));
@@ -341,21 +344,22 @@ int pool_lease_rows(const ProbeEnv& env, const void* owner, uint64_t lo_bytes, u
 
 void pool_release_arena(int device, const void* owner) {
     if (!valid(device)) return;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     release(g_pool[device], owner, false);
 }
 
 void pool_release_rows(int device, const void* owner) {
     if (!valid(device)) return;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     release(g_pool[device], owner, true);
 }
 
 bool pool_trim(int device) {
     if (!valid(device)) return false;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     Pool& p = g_pool[device];
     if (!p.va || !p.leases.empty()) return false;
+    if (hipSetDevice(device) != hipSuccess) { (void)hipGetLastError(); return false; }
     (void)hipDeviceSynchronize();
     free_pair(p);
     return true;
@@ -363,7 +367,7 @@ bool pool_trim(int device) {
 
 bool pool_leased_by(int device, const void* owner, const char* ptr) {
     if (!valid(device)) return false;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     const Pool& p = g_pool[device];
     if (!p.va || ptr < p.va || ptr >= p.va + 2 * p.half) return false;
     const uint64_t off = (uint64_t)(ptr - p.va);
@@ -376,7 +380,7 @@ bool pool_leased_by(int device, const void* owner, const char* ptr) {
 
 SearchRecord pool_record(int device) {
     if (!valid(device)) return SearchRecord{};
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_mutex[device]);
     return g_pool[device].rec;
 }
 

@@ -19,6 +19,12 @@ counted -- moves the same bytes between the same addresses as
     direct      the same for direct: rank 0's and the straggler's whole buffers are read, the sum goes to every rank
     copy/read/write   one buffer copied to another; all buffers read; all buffers written
 
+With 16, 24, ... 64 ranks (--ranks) the mixes are instead
+
+    eights          every rank buffer read and written once, in place, by n/8 jobs of eight ranks each (ranks 8j .. 8j+7):
+                    a ring's traffic over n ranks moved by work items that walk 8 buffers instead of n
+    eights_strided  the same with job j on ranks j, j + n/8, ... (half of them in either region of HBM)
+
 One line per mix: microseconds, GB/s, fraction of the 8 TB/s peak, the fastest shape and the slowest shape's time.
 """
 import argparse
@@ -45,6 +51,14 @@ def mixes(n, chunk, whole, es):
     return [m for m in out if len(m[1]) <= 8 and all(len(rd) <= 8 and len(wr) <= 8 for rd, wr, _ in m[1])]
 
 
+def mixes_many(n, whole):
+    """More than eight ranks: every rank buffer read and written once, in place, by jobs of eight ranks each -- the
+    traffic of a ring over n ranks, moved by work items that walk 8 buffers instead of n."""
+    g = n // 8
+    return [("eights", [(list(range(8 * j, 8 * j + 8)), list(range(8 * j, 8 * j + 8)), 0) for j in range(g)], whole),
+            ("eights_strided", [(list(range(j, n, g)), list(range(j, n, g)), 0) for j in range(g)], whole)]
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--ranks", type=int, default=8)
@@ -56,11 +70,13 @@ def main(argv=None) -> int:
     args = ap.parse_args(argv)
     lib = capi.load_library()
     n = args.ranks
-    if n < 3 or n > 8:
-        print("3 to 8 ranks, please: a probe job holds at most 8 streams a side", file=sys.stderr)
+    if n < 3 or (n > 8 and (n % 8 or n > 64)):
+        print("3 to 8 ranks (a probe job holds at most 8 streams a side), or 16, 24, ... 64 for the mixes of eight ranks per job", file=sys.stderr)
         return 2
     es = capi.ELEM_SIZE[args.dtype]
     nbytes = lib.pad_bytes(int(args.mib * (1 << 20)), n)
+    if n > 8:
+        nbytes -= nbytes % 4096                             # whole buffers are the streams: keep them page-aligned
     chunk = (nbytes // es // (n - 1)) * es
     chunk -= chunk % 16
     ctx = lib.context(0)
@@ -74,7 +90,7 @@ def main(argv=None) -> int:
           % (n, nbytes, args.dtype, chunk, st.arena_spread, capi.SPREAD_REASONS.get(st.spread_reason, "?")))
     print("mix,streams,bytes_moved,us,GB/s,frac_of_8TBps,best_shape(block/vectors/cache_mode/resident/turns),slowest_shape_us,shapes")
     want = [m for m in args.mix.split(",") if m]
-    for name, jobs, size in mixes(n, chunk, nbytes - nbytes % 16, es):
+    for name, jobs, size in (mixes(n, chunk, nbytes - nbytes % 16, es) if n <= 8 else mixes_many(n, nbytes)):
         if want and name not in want:
             continue
         res = ctx.probe_streams(jobs, size, args.reps)
