@@ -7,9 +7,13 @@ are resident in HBM, uniform[-1,1) seeded per rank, pre-work taken as done
 (DELAY = -1 semantics).  Inputs are restored from a device-side snapshot
 before every step, outside the timed region, as the reference re-fills before
 every iteration (by a copy kernel with streaming stores: nothing of the copy
-stays in the caches, neither inputs for the step to find nor modified lines
-for it to push out); each step is timed with HIP events on the executor's
-stream, as the reference times each iteration.
+stays in the caches); then, untimed as well, the same schedule runs on a
+second set of rank buffers, so that the timed step starts where a step in a
+sequence of AllReduces starts: with its predecessor's last stores still in
+the Infinity Cache, to be pushed out at this step's cost, as its own will be
+at the next one's (class Steps; --behind-restore leaves that out).  Each step
+is timed with HIP events on the executor's stream, as the reference times
+each iteration.
 
 value     = bytes that reach memory per step / mean step time: an HBM rate,
             at most the 8 TB/s peak.  The bytes are the plan's of this very
@@ -165,15 +169,48 @@ def live_traffic(args, kernel_pattern, bytes_per_rank):
             "write_kib": round(write, 1), "write_factor": round(wf, 5)}
 
 
-def timed_steps(ctx, steps, warmup):
-    for _ in range(warmup):
-        ctx.restore()
-        ctx.run(-1.0)
-    out = []
-    for _ in range(steps):
-        ctx.restore()                 # untimed: the batch is put back in place, resident in HBM
-        out.append(ctx.run(-1.0))     # start event, the launches, stop event, block on stop
-    return out
+class Steps:
+    """How a step is timed.  Before every timed step the inputs are restored from the device snapshot (untimed, a copy
+    kernel that streams) and then, untimed as well, the same schedule runs on a second set of rank buffers
+    (capi.Predecessor): the timed step starts with what such a step leaves modified in the 256 MB Infinity Cache and
+    pays for pushing it out, as the next step pays for what this one leaves -- the position of a step in a sequence of
+    AllReduces.  Behind the restore alone (`clean`) a step with cached stores is timed 3 to 12 % too fast: the last
+    256 MB it writes are still in the cache when its stop event fires."""
+
+    def __init__(self, ctx, clean):
+        self.ctx, self.clean, self.pred = ctx, clean, None
+        self._shape = None
+
+    def prepare(self, main, prework=None, use_graph=False):
+        self.ctx.prepare(main, prework, use_graph=use_graph)
+        if self.clean:
+            return
+        shape = (self.ctx.n, self.ctx.bytes_per_rank, self.ctx.dtype)
+        if self.pred is None or shape != self._shape:
+            self.drop()
+            self.pred, self._shape = self.ctx.predecessor(), shape
+        self.pred.prepare(main, prework)
+
+    def drop(self):
+        """The second set of rank buffers goes (before the timed context allocates others: both lease from one pool)."""
+        if self.pred is not None:
+            self.pred.close()
+            self.pred = None
+
+    def ready(self):
+        self.ctx.restore()                # untimed: the batch is put back in place, resident in HBM
+        if self.pred is not None:
+            self.pred.run()               # untimed: the step before this one, on buffers of its own
+
+    def timed(self, steps, warmup, delay=-1.0):
+        for _ in range(warmup):
+            self.ready()
+            self.ctx.run(delay)
+        out = []
+        for _ in range(steps):
+            self.ready()
+            out.append(self.ctx.run(delay))     # start event, the launches, stop event, block on stop
+        return out
 
 
 def rates(st, ms):
@@ -190,15 +227,15 @@ def leg_rates(st, ms, fused=False):
             "algorithmic_GBps": round(alg / ms / 1e6, 1)}
 
 
-def other_configs(lib, ctx, orc, many, steps, warmup):
+def other_configs(lib, seq, orc, many, steps, warmup):
     """The BASELINE configurations beside the headline one, each timed by this run on the same device with the same
-    step protocol (inputs restored from the device snapshot before every step, untimed; events on the executor's
-    stream): what the reference binary times for any size, algorithm and delay (allreduce_8GPU.cu:1009-1066,
+    step protocol (class Steps; events on the executor's stream): what the reference binary times for any size, algorithm and delay (allreduce_8GPU.cu:1009-1066,
     reducescatter.cu:88-121).  GBps / frac: bytes that reach memory per step / mean step time, and its share of the
     8 TB/s peak; algorithmic_GBps: every row priced on its own.  ok: all ranks hold the same bits afterwards and, with the
     CPU checker loaded, every element of every rank equals the checker's (null when a check was not made)."""
     import numpy as np
     from oracle import parse_table
+    ctx = seq.ctx
     out = {"legend": "ms: mean step; GBps, frac: bytes that reach memory / ms, of 8 TB/s; ok: ranks identical and every element = CPU checker; "
                      "placed: 1 = ranks in two regions of HBM, else -(SAR_SPREAD_* reason)"}
 
@@ -209,6 +246,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
         return lib.parse(text, n), parse_table(text)
 
     def place(n, nbytes, dtype, fill):
+        seq.drop()
         ctx.set_tuning(**lib.default_tuning().as_dict())
         ctx.alloc_ranks(n, nbytes, dtype)
         for r in range(n):
@@ -221,12 +259,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
         return 1 if st.arena_spread else -int(st.spread_reason)
 
     def steps_ms(delay, k, w):
-        for _ in range(w):
-            ctx.restore(); ctx.run(delay)
-        ts = []
-        for _ in range(k):
-            ctx.restore(); ts.append(ctx.run(delay))
-        return ts
+        return seq.timed(k, w, delay)
 
     def ok(alg, rounds, dtype, delay, n, parts):
         same = bool(ctx.ranks_identical((ctx.elems // parts) * parts))
@@ -248,7 +281,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     nbytes = lib.pad_bytes(1 << 20, n)
     place(n, nbytes, "f32", lambda r: ctx.fill_uniform(r, r, -1.0, 1.0))
     main4, rounds4 = table(n)
-    ctx.prepare(main4, lib.builtin("prework_rs", n))
+    seq.prepare(main4, lib.builtin("prework_rs", n))
     st = ctx.stats()
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
@@ -262,7 +295,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     nbytes = lib.pad_bytes(64 << 20, n)
     place(n, nbytes, "f16", lambda r: ctx.fill_uniform(r, 300 + r, -0.5, 0.5))
     main6, rounds6 = table(n)
-    ctx.prepare(main6, lib.builtin("prework_rs", n))
+    seq.prepare(main6, lib.builtin("prework_rs", n))
     st = ctx.stats()
     ts = steps_ms(0.0, steps, warmup)
     leg = leg_rates(st, statistics.fmean(ts), fused=bool(st.fused_prework))
@@ -282,7 +315,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
         row = {}
         for alg in ("stragglar", "ring", "rhd", "direct"):
             sched = main8 if alg == "stragglar" else lib.builtin(alg, n)
-            ctx.prepare(sched, None)
+            seq.prepare(sched, None)
             st = ctx.stats()
             r = leg_rates(st, statistics.fmean(steps_ms(-1.0, k, w)))
             row[alg] = [round(r["ms"] * 1e3, 2), r["GBps"], r["frac"], ok(alg, rounds8 if alg == "stragglar" else None, "f32", -1.0, n, sched.parts)]
@@ -297,7 +330,7 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
     place(n, nbytes, "bf16", lambda r: ctx.fill_normal(r, 700 + r, 0.0, 1e-3))
     pre8 = lib.builtin("prework_rs", n)
     k, w = max(3, steps // 4), 1
-    ctx.prepare(main8, pre8)
+    seq.prepare(main8, pre8)
     ts = steps_ms(delay, k, w)
     total = statistics.fmean(ts)
     leg = {"what": "%d B per rank, DELAY %.0f ms, pre-work beside the straggler's sleep" % (nbytes, delay),
@@ -305,13 +338,13 @@ def other_configs(lib, ctx, orc, many, steps, warmup):
            "reference_style_GiBps": round(nbytes / 2.0 ** 30 * 1000.0 / (total - delay), 2), "placed": placed(),
            "ok": ok("stragglar", rounds8, "bf16", delay, n, n - 1)}
     # the two kernels of that run, each on its own: bytes that reach memory / time of the launch
-    ctx.prepare(main8, None)
+    seq.prepare(main8, None)
     st = ctx.stats()
     kms = []
     for _ in range(k + w):
-        ctx.restore(); kms.append(sum(ctx.run_profiled()))
+        seq.ready(); kms.append(sum(ctx.run_profiled()))
     leg["schedule_kernel"] = leg_rates(st, statistics.fmean(kms[w:]))
-    ctx.prepare(pre8, None)
+    seq.prepare(pre8, None)
     st = ctx.stats()
     leg["prework_kernel"] = leg_rates(st, statistics.fmean(steps_ms(-1.0, k, w)))
     out["config2_n8_1GiB_bf16_delay5ms"] = leg
@@ -332,6 +365,8 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true", help="skip the legs for the BASELINE configurations beside the headline one (n=4 1 MiB, n=6 fp16 with "
                     "pre-work, the message-size sweep, bf16 1 GiB with DELAY = 5 ms)")
     ap.add_argument("--no-live-traffic", action="store_true", help="do not run the two rocprofv3 --pmc child runs that measure roofline.traffic; use the figure kept under profiles/")
+    ap.add_argument("--behind-restore", action="store_true", help="time every step behind the restore alone (clean Infinity Cache) instead of behind "
+                    "the same step on a second set of rank buffers; flatters steps with cached stores")
     ap.add_argument("--traffic-child", action="store_true", help=argparse.SUPPRESS)      # a run of this script under the profiler: headline steps only
     ap.add_argument("--graph", action="store_true", help="replay the rounds as one hipGraph (slower than eager launches on this stack)")
     ap.add_argument("--executor", type=int, default=None, choices=[0, 1, 2],
@@ -375,13 +410,15 @@ def main():
     ctx.snapshot()
     if overrides:
         ctx.set_tuning(**overrides)
-    ctx.prepare(main_sched, None, use_graph=args.graph)
+    seq = Steps(ctx, args.behind_restore)
+    seq.prepare(main_sched, None, use_graph=args.graph)
     st = ctx.stats()
     tune = ctx.get_tuning().as_dict()
 
-    step_ms = timed_steps(ctx, args.steps, args.warmup)
+    step_ms = seq.timed(args.steps, args.warmup)
     identical = ctx.ranks_identical((elems // main_sched.parts) * main_sched.parts)
     if args.traffic_child:
+        seq.drop()
         ctx.close()
         return
     ms = statistics.fmean(step_ms)
@@ -399,9 +436,9 @@ def main():
     launch_bytes = ctx.launch_bytes()
     per_launch = [0.0] * len(launch_bytes)
     reps = max(3, min(10, args.steps))
-    ctx.prepare(main_sched, None, use_graph=False)
+    seq.prepare(main_sched, None, use_graph=False)
     for _ in range(reps):
-        ctx.restore()
+        seq.ready()
         for i, t in enumerate(ctx.run_profiled()):
             per_launch[i] += t / reps
     mean_launch_ms = statistics.fmean(per_launch)
@@ -447,6 +484,7 @@ def main():
                                "DELAY=-1, %d ranks resident in one GPU's HBM; value = bytes that reach memory per step / step time "
                                "(an HBM rate; the rows' algorithmic bytes / step time is algorithmic_GBps)" % (n, args.alg, table_name, args.mib, nbytes, n),
                    "ranks": n, "bytes_per_rank": nbytes, "algorithm": args.alg, "graph": bool(args.graph),
+                   "timed": "every step behind the restore alone (clean cache)" if args.behind_restore else "every step behind the same step on a second set of rank buffers (as in a sequence of AllReduces)",
                    "tuning": "library defaults" if tune == lib.default_tuning().as_dict() else tune, "executor_used": "column" if st.executor == 1 else "rounds"},
         "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
         "memory_bytes_per_step": int(to_memory),
@@ -469,8 +507,8 @@ def main():
     if st.col_slots and args.forward is None:
         # the same steps with every operand loaded from the rank buffers
         ctx.set_tuning(col_forward=0)
-        ctx.prepare(main_sched, None, use_graph=args.graph)
-        plain_ms = timed_steps(ctx, args.steps, args.warmup)
+        seq.prepare(main_sched, None, use_graph=args.graph)
+        plain_ms = seq.timed(args.steps, args.warmup)
         pm = statistics.fmean(plain_ms)
         leg = {"algorithmic_GBps": round(st.algorithmic_bytes / pm / 1e6, 1), "unit": "GB/s", "ms_per_step": round(pm, 5),
                "algorithmic_frac": round(st.algorithmic_bytes / pm / 1e6 / HBM_PEAK_GBPS, 4),
@@ -485,7 +523,7 @@ def main():
             leg["frac_of_hbm_peak"] = round(leg["memory_side_GBps"] / HBM_PEAK_GBPS, 4)
         rec["every_operand_loaded"] = leg
         ctx.set_tuning(col_forward=1)
-        ctx.prepare(main_sched, None, use_graph=False)
+        seq.prepare(main_sched, None, use_graph=False)
 
     if args.alg == "stragglar" and st.col_slots and 2 <= n - 1 <= 8:
         # What the memory system delivers for this kernel's own mix of streams, by a kernel that does nothing else
@@ -506,9 +544,9 @@ def main():
         # cold reads and two writes per element, in place: nothing to forward, so these bytes all reach memory.
         rows = "sar-rows %d %d\n" % (n, n - 1) + "".join("round\nxreduce %d %d %d\n" % (r, n - 1, r) for r in range(n - 1))
         xsched = lib.parse(rows, n)
-        ctx.prepare(xsched, None, use_graph=args.graph)
+        seq.prepare(xsched, None, use_graph=args.graph)
         xst = ctx.stats()
-        xms = timed_steps(ctx, args.steps, args.warmup)
+        xms = seq.timed(args.steps, args.warmup)
         xm = statistics.fmean(xms)
         xmem, xhbm, _ = rates(xst, xm)
         rec["reduce_steps_alone"] = {"rows": "%d exchanges (XREDUCE) of one chunk each, no copies" % (n - 1), "ms_per_step": round(xm, 5),
@@ -521,7 +559,7 @@ def main():
             rec["reduce_steps_alone"]["stream_ceiling_GBps"] = round(res.gbps, 1)
             rec["reduce_steps_alone"]["vs_ceiling"] = round(xhbm / res.gbps, 4)
         ctx.restore()
-        ctx.prepare(main_sched, None, use_graph=False)
+        seq.prepare(main_sched, None, use_graph=False)
 
     orc = inputs = None
     if not args.no_cpu:
@@ -563,9 +601,9 @@ def main():
             if alg == "direct" and n % 2:
                 continue
             sched = lib.builtin(alg, n)
-            ctx.prepare(sched, None, use_graph=args.graph)
+            seq.prepare(sched, None, use_graph=args.graph)
             cst = ctx.stats()
-            cms = timed_steps(ctx, args.steps, args.warmup)
+            cms = seq.timed(args.steps, args.warmup)
             cm = statistics.fmean(cms)
             cmem, chbm, calg = rates(cst, cm)
             leg = {"ms_per_step": round(cm, 5), "ms_per_step_min": round(min(cms), 5),
@@ -580,8 +618,9 @@ def main():
         rec["comparators"] = comps
     if not args.no_other_configs and not args.no_comparators and args.alg == "stragglar" and n == 8 and args.mib == 256 and not args.graph and not overrides:
         t0 = time.perf_counter()
-        rec["other_configs"] = other_configs(lib, ctx, orc, many, args.steps, args.warmup)
+        rec["other_configs"] = other_configs(lib, seq, orc, many, args.steps, args.warmup)
         rec["other_configs"]["seconds"] = round(time.perf_counter() - t0, 1)
+    seq.drop()
     ctx.close()
     print(json.dumps(rec))
     bad = not identical or rec.get("bit_exact_vs_cpu_checker") is False

@@ -123,7 +123,11 @@ typedef struct sar_tuning_t {
                           /*     loads and cached stores, 2 = planned (default).  One launch per     */
                           /*     round plans per row: streaming unless the data is read again within */
                           /*     `reuse_rounds`.  The column executor has one policy per launch: it  */
-                          /*     plans streaming loads when every re-read is forwarded, else cached  */
+                          /*     plans streaming loads when every re-read is forwarded (else all     */
+                          /*     cached), and streaming stores as well once the rank buffers add up  */
+                          /*     to 512 MiB and more: a cached store is only paid for when the line  */
+                          /*     is pushed out of the 256 MB Infinity Cache, by this launch or the   */
+                          /*     next, and in a sequence of steps streaming stores are 1 - 3 % ahead */
     int32_t reuse_rounds; /* look-ahead of policy 2, in rounds                                       */
     int32_t reverse_odd;  /* 1 = odd rounds walk their tiles backwards (keeps the cache tail warm)   */
     int32_t segments;     /* >1: cut every row into this many pieces and run the whole schedule      */

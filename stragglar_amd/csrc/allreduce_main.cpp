@@ -22,6 +22,11 @@
 //                      the 8 TB/s HBM peak, and the rows' algorithmic bytes and rate
 //   --executor 0|1|2   0 = one launch per round, 1 = the column kernel (one launch per schedule), 2 = the library's
 //                      choice (default)
+//   --sequence 0|1     1 (default): every timed iteration runs directly behind the same step on a second set of rank
+//                      buffers (untimed), as in a sequence of AllReduces: it starts with that step's last stores still
+//                      in the 256 MB Infinity Cache and pays for pushing them out, as the next would for its own.
+//                      0: behind the fill alone, as the reference times it (its GPUs have no such cache; here a step
+//                      with cached stores is then timed 3 to 12 % too fast)
 //   --nocheck          skip the final "all ranks hold the same" check: for a --schedule that times a part of a
 //                      table (a row list of the exchanges alone, say) and is no AllReduce
 #include <cerrno>
@@ -94,7 +99,7 @@ int main(int argc, char* argv[]) {
     int numIters = atoi(argv[3]);
     float sleepTime = (float)atof(argv[4]);
 
-    int numRanks = 8, dtype = SAR_F32, use_graph = 0, base = -1, report = 0, executor = -1, check = 1;
+    int numRanks = 8, dtype = SAR_F32, use_graph = 0, base = -1, report = 0, executor = -1, check = 1, sequence = 1;
     unsigned long long seed = 0;
     std::string schedule_path, init = "reference";
     for (int i = 5; i < argc; ++i) {
@@ -116,6 +121,7 @@ int main(int argc, char* argv[]) {
         else if (a == "--graph") use_graph = atoi(need("--graph"));
         else if (a == "--report") report = 1;
         else if (a == "--executor") executor = atoi(need("--executor"));      // 0 one launch per round, 1 column kernel, 2 the library's choice
+        else if (a == "--sequence") sequence = atoi(need("--sequence"));
         else if (a == "--nocheck") check = 0;                                  // a --schedule that is not an AllReduce (timing parts of a table)
         else { fprintf(stderr, "Unknown option: %s\n", a.c_str()); exit(EXIT_FAILURE); }
     }
@@ -186,6 +192,28 @@ int main(int argc, char* argv[]) {
     sar_stats_t st;
     CHECK_SAR(sar_stats(ctx, &st));
 
+    // the step before every timed one, on rank buffers of its own (--sequence)
+    sar_ctx* before = NULL;
+    if (sequence) {
+        CHECK_SAR(sar_create(0, &before));
+        sar_tuning_t tune;
+        CHECK_SAR(sar_get_tuning(ctx, &tune));
+        CHECK_SAR(sar_set_tuning(before, &tune));
+        if (sar_alloc_ranks(before, numRanks, (uint64_t)size * es, dtype) != SAR_OK) {
+            fprintf(stderr, "no room for a second set of rank buffers (%s): every iteration is timed behind the fill alone\n", sar_last_error());
+            sar_destroy(before); before = NULL;
+        } else {
+            CHECK_SAR(sar_prepare(before, prework, main_sched, 0));
+        }
+    }
+    int before_runs = 0;
+    auto step_before = [&]() {
+        if (!before) return;
+        if (before_runs++ % 8 == 0)                      // sums of sums grow: fresh values before they overflow
+            for (int r = 0; r < numRanks; ++r) CHECK_SAR(sar_fill_uniform(before, r, 101 + r, -6e-5, 6e-5));
+        CHECK_SAR(sar_run(before, prework ? 0.f : -1.f, NULL));
+    };
+
     auto fill = [&]() {
         if (init == "reference") { CHECK_SAR(sar_fill_reference_pattern(ctx, alg, sleepTime, base)); return; }
         for (int r = 0; r < numRanks; ++r) {
@@ -202,6 +230,7 @@ int main(int argc, char* argv[]) {
     double sum_ms = 0; double min_ms = 1e30;
     for (int iter = 0; iter < numIters + 1; ++iter) {
         fill();
+        step_before();
         float ms = 0.f;
         CHECK_SAR(sar_run(ctx, sleepTime, &ms));
         if (iter == 0) continue;
@@ -263,6 +292,7 @@ int main(int argc, char* argv[]) {
 
     sar_schedule_free(main_sched);
     sar_schedule_free(prework);
+    sar_destroy(before);
     sar_destroy(ctx);
     for (int i = 0; i < numRanks; ++i) printf("Rank %d, done\n", i);
     return (failures && init != "reference") ? EXIT_FAILURE : 0;

@@ -689,19 +689,29 @@ private:
         // Cache policy of the launch (the column kernel takes one for all its rows).  Planned (2): when every re-read is
         // forwarded, what is still loaded is read exactly once: streaming loads (+1.5 % for the StragglAR table);
         // otherwise the re-reads are meant to find their data in the caches and nothing streams (streaming loads cost
-        // 4-10 % there).  Streaming stores never paid in this kernel (-3 to -25 %).
+        // 4-10 % there).
         // A launch in which no row reads what another wrote or read (the exchanges of a table on their own, a pre-work
-        // on its own) has nothing to find in the caches either: streaming loads (seven exchanges of 256 MiB ranks,
-        // n = 8: 161 against 171 us).  When all its rows are multi-source rows, streaming stores as well: seven reads
-        // and one write per vector run 3 % faster with them (358 against 369 us), and a pre-work that runs beside the
-        // straggler's delay then leaves no modified lines in the Infinity Cache for the schedule to push out (n = 8,
-        // 1 GiB per rank: the schedule took 65 us longer behind a pre-work with cached stores).
+        // on its own) has nothing to find in the caches either: streaming loads.  When all its rows are multi-source
+        // rows, streaming stores as well: seven reads and one write per vector run 3 % faster with them (358 against
+        // 369 us), and a pre-work that runs beside the straggler's delay then leaves no modified lines in the Infinity
+        // Cache for the schedule to push out (n = 8, 1 GiB per rank: the schedule took 65 us longer behind a pre-work
+        // with cached stores).
+        // Streaming stores for every such plan once the payload is twice the Infinity Cache and more: a cached store
+        // is fast while the cache takes it and is paid for when the line is pushed out, by this launch or the next.
+        // Timed behind a restore that leaves the cache clean, cached stores look 3 to 12 % faster than they are (the
+        // last 256 MB of the launch never reach memory inside the timed span); timed in a sequence of steps, each
+        // inheriting what the one before left, streaming stores win: n = 8, 256 MiB per rank, ring 680 against 703 us,
+        // halving-doubling 694 against 714, the exchanges alone 175 against 177 (1 GiB: 698 against 722); 64 MiB per
+        // rank: ring 174 against 180, StragglAR 106.5 against 108.5.  Up to 32 MiB per rank (everything fits the
+        // cache and the next step finds it there) cached stores stay ahead by 1 to 5 %.
         const int cp = env_.tune.cache_policy;
         bool only_multi_source = !cr_.empty();
         for (const auto& r : cr_) only_multi_source = only_multi_source && r.d.kind == SAR_OP_MREDUCE;
-        // A plan that mostly stores, one vector per lane, payload far beyond the Infinity Cache (choose_vectors): streaming
-        // stores as well, there is no use in keeping lines that nobody reads again.
-        const uint32_t planned = all_found_ ? (store_heavy_ && !plan_.two_vectors ? 2u : 1u) : no_reuse_ ? (only_multi_source ? 2u : 1u) : 0u;
+        const bool beyond_cache = env_.bytes_per_rank * (uint64_t)env_.n >= (512ull << 20);
+        // (A plan that mostly stores, one vector per lane, payload far beyond the cache -- choose_vectors -- streamed its
+        // stores before this rule and still does.)
+        const uint32_t planned = all_found_ ? (beyond_cache || (store_heavy_ && !plan_.two_vectors) ? 2u : 1u)
+                                            : no_reuse_ ? (only_multi_source || beyond_cache ? 2u : 1u) : 0u;
         plan_.policy = cp == 0 ? 0u : cp == 1 ? 2u : cp == 3 ? 1u : planned;
 
         // Dispatch order of the items.  All columns of one component before the next component keeps the resident

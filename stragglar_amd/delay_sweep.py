@@ -9,7 +9,9 @@ reference's benchmark runs it in delay mode (stragglar_allreduce_delay and its
 siblings, stragglar/allreduce_8GPU.cu:115-137,201-219,535-553,876-898): the
 straggler's stream sleeps DELAY ms; meanwhile StragglAR's other ranks do their
 ReduceScatter pre-work and `direct`'s do their (n-1)-rank AllReduce, ring and
-rhd can only wait.  Printed per row, in the reference's CSV convention:
+rhd can only wait.  Every timed run follows the same step (without the delay) on a
+second set of rank buffers, as in a sequence of AllReduces (capi.Predecessor).
+Printed per row, in the reference's CSV convention:
 
     algorithm,buffer_size_bytes,delay,runtime_ms,runtime_minus_delay_ms,BW(GB/s)
 
@@ -47,6 +49,7 @@ def main(argv=None) -> int:
     for r in range(n):
         ctx.fill_uniform(r, 7 + r, -1.0, 1.0)
     ctx.snapshot()
+    pred = ctx.predecessor()
     print("algorithm,buffer_size_bytes,delay,runtime_ms,runtime_minus_delay_ms,BW(GB/s)")
     net = {}
     for alg in algs:
@@ -60,10 +63,12 @@ def main(argv=None) -> int:
             main_sched = lib.builtin(alg, n)
             prework = lib.builtin("prework_ar", n) if alg == "direct" else None
         ctx.prepare(main_sched, prework)
+        pred.prepare(main_sched, prework)
         for d in delays:
             ts = []
             for it in range(args.iters + 1):
                 ctx.restore()
+                pred.run()
                 ms = ctx.run(d)
                 if it:
                     ts.append(ms)
@@ -71,6 +76,7 @@ def main(argv=None) -> int:
             rest = ms - (d if d > 0 else 0.0)
             net[(alg, d)] = rest
             print("%s,%d,%.3f,%.3f,%.3f,%.3f" % (alg, nbytes, d, ms, rest, nbytes / 2 ** 30 * 1000 / rest))
+    pred.close()
     ctx.close()
     if "ring" in algs:
         print("# milliseconds saved against ring after the straggler has arrived (positive = finishes sooner)")

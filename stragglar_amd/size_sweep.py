@@ -6,7 +6,9 @@
 
 For every size (bytes per rank before padding; padded as pad_buffers.py pads) and algorithm the emulated AllReduce runs
 as the reference's benchmark runs it with DELAY = -1 (allreduce_8GPU.cu:1029-1047: the same four algorithms at any
-size), the inputs restored before every iteration, eagerly launched and as a replayed hipGraph.  One CSV line each:
+size), the inputs restored before every iteration and the timed step directly behind the same step on a second set of rank
+buffers (capi.Predecessor: the position of a step in a sequence of AllReduces), eagerly launched and as a replayed
+hipGraph.  One CSV line each:
 
     algorithm,bytes_per_rank,graph,launches,executor,median_us,min_us,memory_GBps,algorithmic_GBps,host_call_us
 
@@ -46,6 +48,7 @@ def main(argv=None) -> int:
         for r in range(n):
             ctx.fill_uniform(r, 11 + r, -1.0, 1.0)
         ctx.snapshot()
+        pred = ctx.predecessor()
         for alg in [a for a in args.algs.split(",") if a]:
             if alg == "stragglar":
                 path = os.path.join(HERE, "schedules", "stragglar_n%d.txt" % n)
@@ -56,10 +59,12 @@ def main(argv=None) -> int:
                 sched = lib.builtin(alg, n)
             for graph in (0, 1):
                 ctx.prepare(sched, None, use_graph=bool(graph))
+                pred.prepare(sched, None)
                 st = ctx.stats()
                 ts, host = [], []
                 for it in range(args.iters + 2):
                     ctx.restore()
+                    pred.run()
                     t0 = time.perf_counter()
                     ms = ctx.run(-1.0)
                     t1 = time.perf_counter()
@@ -71,6 +76,7 @@ def main(argv=None) -> int:
                 print("%s,%d,%d,%d,%s,%.2f,%.2f,%.0f,%.0f,%.1f" % (alg, nbytes, graph, st.launches, "column" if st.executor else "rounds",
                                                                   med * 1e3, min(ts) * 1e3, to_memory / med / 1e6, st.algorithmic_bytes / med / 1e6,
                                                                   statistics.median(host) * 1e6), flush=True)
+        pred.close()                          # before the next size: both sets of rank buffers lease from one pool
     ctx.close()
     return 0
 

@@ -13,6 +13,10 @@ a pre-work collective on its own (prework_rs: reducescatter.cu:103-108); --sched
 file instead.  Every --vary NAME=V1,V2,... names a field of sar_tuning_t; the grid is their product, the first value
 of each being the base line.
 
+Every timed step runs directly behind the same schedule on a second set of rank buffers (capi.Predecessor), as in a
+sequence of AllReduces: it starts with what such a step leaves modified in the Infinity Cache and pays for it, as its
+own leftovers are paid for by the next (--behind-restore times each step behind the streaming restore alone).
+
 CSV: the varied fields, the executor and column width in use, median and fastest step in microseconds, the bytes that
 reach memory per step, their rate in GB/s and as a fraction of the 8 TB/s peak, and whether all ranks hold the same
 bits afterwards (for schedules that are an AllReduce).
@@ -36,6 +40,7 @@ def main(argv=None) -> int:
     ap.add_argument("--mib", type=float, default=256.0, help="unpadded MiB per rank")
     ap.add_argument("--dtype", default="f32", choices=sorted(capi.DTYPES))
     ap.add_argument("--iters", type=int, default=9, help="timed steps per setting (the first two are dropped)")
+    ap.add_argument("--behind-restore", action="store_true", help="no predecessor step: every timed step starts with a clean cache")
     ap.add_argument("--vary", action="append", default=[], metavar="NAME=V1,V2", help="a tuning field and the values to try")
     args = ap.parse_args(argv)
     lib = capi.load_library()
@@ -81,10 +86,15 @@ def main(argv=None) -> int:
         ctx.set_tuning(**t)
         ctx.prepare(sched, None)
         st = ctx.stats()
+        pred = None if args.behind_restore else ctx.predecessor(sched)
         ts = []
         for _ in range(max(3, args.iters)):
             ctx.restore()
+            if pred:
+                pred.run()
             ts.append(ctx.run(-1.0))
+        if pred:
+            pred.close()
         same = ctx.ranks_identical((ctx.elems // sched.parts) * sched.parts) if allreduce else ""
         ts = sorted(ts[2:])
         med = ts[len(ts) // 2]
