@@ -197,18 +197,18 @@ class Steps:
             self.pred.close()
             self.pred = None
 
-    def ready(self):
+    def ready(self, delay=-1.0):
         self.ctx.restore()                # untimed: the batch is put back in place, resident in HBM
         if self.pred is not None:
-            self.pred.run()               # untimed: the step before this one, on buffers of its own
+            self.pred.run(delay)          # untimed: the step before this one, on buffers of its own
 
     def timed(self, steps, warmup, delay=-1.0):
         for _ in range(warmup):
-            self.ready()
+            self.ready(delay)
             self.ctx.run(delay)
         out = []
         for _ in range(steps):
-            self.ready()
+            self.ready(delay)
             out.append(self.ctx.run(delay))     # start event, the launches, stop event, block on stop
         return out
 

@@ -374,7 +374,9 @@ class Predecessor:
         self.ctx.prepare(main, prework)
         self._with_prework = prework is not None
 
-    def run(self):
+    def run(self, delay_ms: Optional[float] = None):
+        """One untimed step; `delay_ms` as for the timed step that follows (default: 0 with a pre-work, else -1), so that
+        the same launches run."""
         if self._runs % 8 == 0:                       # sums of sums grow: fresh values before they overflow
             for r in range(self.ctx.n):
                 if self.ctx.dtype == "f32":
@@ -382,7 +384,7 @@ class Predecessor:
                 else:
                     self.ctx.fill_uniform(r, 101 + r, -2.0 ** -14, 2.0 ** -14)
         self._runs += 1
-        self.ctx.run(0.0 if self._with_prework else -1.0)
+        self.ctx.run((0.0 if self._with_prework else -1.0) if delay_ms is None else delay_ms)
 
     def close(self):
         self.ctx.close()

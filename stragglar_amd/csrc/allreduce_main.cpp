@@ -211,7 +211,7 @@ int main(int argc, char* argv[]) {
         if (!before) return;
         if (before_runs++ % 8 == 0)                      // sums of sums grow: fresh values before they overflow
             for (int r = 0; r < numRanks; ++r) CHECK_SAR(sar_fill_uniform(before, r, 101 + r, -6e-5, 6e-5));
-        CHECK_SAR(sar_run(before, prework ? 0.f : -1.f, NULL));
+        CHECK_SAR(sar_run(before, sleepTime, NULL));      // the same launches as the timed step
     };
 
     auto fill = [&]() {

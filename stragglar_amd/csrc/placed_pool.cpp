@@ -194,7 +194,10 @@ int find_pair(const ProbeEnv& env, uint64_t half, Pool& p) {
     char* hi = nullptr;
     for (int round = 0; round < 4 && !hi; ++round) {
         const int k = times.empty() ? -1 : spread_pick(same, times.data(), (int)times.size());
-        if (k < 0) break;
+        if (k < 0) {
+            if (debug) std::fprintf(stderr, "sar spread: no verdict on %zu candidates (nobody clearly below the yardstick, or no gap between those and the rest)\n", times.size());
+            break;
+        }
         char* cand = live[first_cand + (size_t)k].va;
         const float t2 = probe_ms(env, stamps, lo + half - window, cand + half - window, 3);
         if (debug) std::fprintf(stderr, "sar spread: candidate %d picked (%.1f us), other windows %.1f us\n", k + 1, times[(size_t)k] * 1e3, t2 * 1e3);
@@ -243,7 +246,15 @@ int ensure_pair(const ProbeEnv& env, Pool& p, uint64_t need) {
     if (p.va) { (void)hipDeviceSynchronize(); free_pair(p); }
     uint64_t half = kMinHalf;
     while (half < need) half <<= 1;
-    return find_pair(env, half, p);
+    // room for a second context of the same shape (a step and its predecessor on buffers of their own, two groups of one
+    // process) where the largest pair allows it: the pair cannot grow while somebody holds a lease
+    const uint64_t least = half;
+    if (half < 2 * need && 2 * half <= kMaxHalf) half <<= 1;
+    int reason = find_pair(env, half, p);
+    // no clear verdict with the larger allocations: the search again with the smaller ones, which the driver cuts from
+    // memory differently
+    if (reason == SAR_SPREAD_NO_PAIR && half > least) reason = find_pair(env, least, p);
+    return reason;
 }
 
 // When a context goes, a pair larger than the smallest one is not kept idle for those that stay.

@@ -9,7 +9,7 @@ reference's benchmark runs it in delay mode (stragglar_allreduce_delay and its
 siblings, stragglar/allreduce_8GPU.cu:115-137,201-219,535-553,876-898): the
 straggler's stream sleeps DELAY ms; meanwhile StragglAR's other ranks do their
 ReduceScatter pre-work and `direct`'s do their (n-1)-rank AllReduce, ring and
-rhd can only wait.  Every timed run follows the same step (without the delay) on a
+rhd can only wait.  Every timed run follows the same step on a
 second set of rank buffers, as in a sequence of AllReduces (capi.Predecessor).
 Printed per row, in the reference's CSV convention:
 
@@ -68,7 +68,7 @@ def main(argv=None) -> int:
             ts = []
             for it in range(args.iters + 1):
                 ctx.restore()
-                pred.run()
+                pred.run(d)
                 ms = ctx.run(d)
                 if it:
                     ts.append(ms)

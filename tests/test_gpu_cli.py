@@ -219,7 +219,21 @@ def test_cli_runs_a_row_list_that_is_no_allreduce():
     assert p.returncode != 0 and "Rank buffers differ" in p.stdout
 
 
-@pytest.mark.parametrize("extra", [[], ["--executor", "0", "--no-live-traffic"], ["--forward", "0", "--no-live-traffic"], ["--alg", "ring", "--no-cpu", "--no-live-traffic"]])
+def test_cli_times_a_step_in_a_sequence_or_behind_the_fill():
+    """--sequence 1 (default): every timed iteration follows the same step on a second set of rank buffers; --sequence 0: the
+    fill alone, as the reference times it.  Same CSV, same result either way; the reference pattern still sums to 36."""
+    for seq in ("1", "0"):
+        p = run(os.path.join(BIN, "allreduce"), "1053696", "stragglar", "3", "-1", "--sequence", seq, "--report")
+        assert p.returncode == 0, p.stdout + p.stderr
+        rows = [l for l in p.stdout.splitlines() if l.startswith("stragglar,")]
+        assert len(rows) == 3 and all(float(r.split(",")[4]) > 0 for r in rows)
+        assert "bytes_to_memory=" in p.stderr
+    p = run(os.path.join(BIN, "allreduce"), "1053696", "stragglar", "2", "0.5", "--sequence", "1")      # the predecessor sleeps as well
+    assert p.returncode == 0 and all(float(r.split(",")[4]) > 0.5 for r in p.stdout.splitlines() if r.startswith("stragglar,")), p.stdout + p.stderr
+
+
+@pytest.mark.parametrize("extra", [[], ["--executor", "0", "--no-live-traffic"], ["--forward", "0", "--no-live-traffic"], ["--alg", "ring", "--no-cpu", "--no-live-traffic"],
+                                   ["--behind-restore", "--no-cpu", "--no-live-traffic"]])
 def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     """bench.py end to end (at 16 MiB per rank so that it takes a second): exactly one JSON line on stdout, the
     keys the harness reads, a roofline object and, for the StragglAR run, the CPU baseline."""
@@ -245,6 +259,7 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     assert rec["memory_bytes_per_step"] == rec["algorithmic_bytes_per_step"] - rec["forwarded_bytes_per_step"] - rec["elided_store_bytes_per_step"]
     assert abs(roof["achieved"] - roof["memory_bytes_per_launch"] / roof["mean_launch_ms"] / 1e6) <= 0.002 * roof["achieved"]
     assert rec["host"]["logical_cpus"] >= 1
+    assert ("restore alone" in rec["config"]["timed"]) == ("--behind-restore" in extra)
     if "--no-live-traffic" not in extra:
         import shutil
         if shutil.which("rocprofv3"):
@@ -252,7 +267,7 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
             # (at this size the rank buffers fit the Infinity Cache, which sits behind the counters)
             assert roof["traffic_source"].startswith("this run"), roof["traffic_source"]
             assert 0.98 <= roof["traffic_vs_plan"] <= 1.02, roof
-    if "--alg" not in extra:
+    if "--alg" not in extra and "--no-cpu" not in extra:
         red = rec["reduce_steps_alone"]
         assert red["memory_bytes_per_step"] == rec["algorithmic_bytes_per_step"] // 4 and red["GBps"] > 0       # 4 S of the 16 S
         assert sorted(rec["comparators"]) == ["direct", "rhd", "ring"]
@@ -324,7 +339,7 @@ def test_tuning_sweep_and_placement_mixes_tools():
     assert [(r[0], r[1]) for r in rows] == [("1", "0"), ("1", "256"), ("2", "0"), ("2", "256")]
     assert all(r[-1] == "True" and float(r[5]) >= float(r[6]) > 0 for r in rows)
     p = run(sys.executable, "-m", "stragglar_amd.tuning_sweep", "--schedule", os.path.join(ROOT, "stragglar_amd", "schedules", "exchanges_n8.rows"),
-            "--mib", "4", "--iters", "3", "--vary", "cache_policy=2,1")
+            "--mib", "4", "--iters", "3", "--vary", "cache_policy=2,1", "--behind-restore")
     assert p.returncode == 0 and len([l for l in p.stdout.splitlines() if l.startswith(("2,", "1,"))]) == 2, p.stdout + p.stderr
     assert run(sys.executable, "-m", "stragglar_amd.tuning_sweep", "--vary", "no_such_field=1").returncode == 2
     p = run(sys.executable, "-m", "stragglar_amd.hbm_regions", "--mixes", "--gib", "32", "--slot-gib", "1", "--per-rank-mib", "64", "--stream-mib", "64")

@@ -520,6 +520,11 @@ _RECORDED_SEARCHES = [
     # allocation reads 175 / 174 us, and candidates elsewhere come first, in between and last
     ((175.2, 209.9, 202.9), 186.0, (211.5, 193.2, 194.0, 206.3, 215.6, 192.9), (163.0, 162.2, 164.0, 163.1, 162.1, 161.9, 162.5, 166.5)),
     ((173.6, 204.0, 217.6), 185.7, (197.9, 191.1, 217.6, 188.3, 193.3, 209.8, 203.4, 188.0), (160.4, 161.2, 166.7, 162.4, 164.4)),
+    # 16 GiB candidates in cut-up memory: the two ends of the first allocation slower than its neighbouring windows (the
+    # median neighbour is the yardstick then), and one candidate in between the populations (0.954 of the yardstick)
+    ((170.9, 190.9, 194.3), 206.0, (182.1, 199.5, 190.2, 202.4), (164.2, 162.0, 163.5)),
+    ((182.5, 202.9, 203.6), 185.8, (191.0, 188.4, 185.9, 189.3, 201.1, 205.7, 200.4, 201.9, 186.0, 190.2, 192.4, 189.5, 196.0, 218.3, 208.5, 204.4,
+                                   191.7, 187.6, 187.9, 189.3, 214.7, 204.8), (159.4, 164.2, 158.8)),
 ]
 
 
