@@ -415,9 +415,10 @@ int sar_probe_streams(sar_ctx* ctx, int njobs, const sar_probe_job* jobs, uint64
 int sar_spread_yardstick(const float* neighbours_ms, float ends_ms, float* yardstick_ms);
 int sar_spread_is_elsewhere(float yardstick_ms, float probe_ms);
 /* The verdict on a whole search: probe_ms[0..n) are the candidates' times against the first allocation.  Returns 1 and
- * *pick = the candidate to take (the fastest) when the times fall into two populations -- candidates elsewhere, clearly
- * below the yardstick, and the rest, with a clear gap between the two in the candidates' own times --, else 0 and *pick = -1:
- * the ranks then sit in one ordinary allocation (SAR_SPREAD_NO_PAIR).  Times <= 0 are failed probes and say nothing. */
+ * *pick = the candidate to take (the fastest) when it is clearly below the yardstick and the times fall into two
+ * populations -- sorted, they jump by 4 % and more somewhere below the limit -- or all lie clearly below the yardstick;
+ * else 0 and *pick = -1: the ranks then sit in one ordinary allocation (SAR_SPREAD_NO_PAIR).  Times <= 0 are failed
+ * probes and say nothing. */
 int sar_spread_pick(float yardstick_ms, const float* probe_ms, int n, int* pick);
 
 /* Ticks of the device's constant-rate wall clock that delay_ms lasts: the

@@ -27,8 +27,8 @@ constexpr uint64_t kProbeStream = 128ull << 20;        // region probe: 8 stream
 // and drifts: in an allocation pieced together from freed memory one neighbouring pair read 173-175 us, which pulled
 // candidates elsewhere at 162-167 us above the limit.  Against the yardstick candidates elsewhere come in at 0.85-0.90
 // on an empty device and 0.932 with 80 GiB of other allocations around, candidates of the same region at 0.98 and more.
-// The candidates' own times must show the gap as well: at least kGap between the slowest "elsewhere" and the fastest
-// other candidate (measured 11-18 %).
+// The candidates' own times must show the two populations as well: sorted, they jump by kGap and more somewhere below
+// the limit (measured 9-18 % between the slowest candidate elsewhere and the fastest of the first allocation's region).
 constexpr float kFaster = 0.95f, kGap = 0.04f;
 constexpr float kStraddle = 0.86f;                     // the two ends of an allocation against its neighbouring windows: below this a
                                                        // boundary runs through it (measured 0.80 with a boundary, 0.90 to 0.93 without)
@@ -281,23 +281,24 @@ bool spread_is_elsewhere(float yardstick_ms, float probe_ms_value) { return prob
 
 int spread_pick(float yardstick_ms, const float* t, int n) {
     if (!(yardstick_ms > 0.f) || !t || n < 1) return -1;
-    // the candidates clearly below the yardstick, and the fastest of the rest
-    int best = -1;
-    float slowest_elsewhere = 0.f, fastest_other = 0.f;
-    for (int i = 0; i < n; ++i) {
-        if (!(t[i] > 0.f)) continue;                                  // a failed probe says nothing
-        if (spread_is_elsewhere(yardstick_ms, t[i])) {
-            slowest_elsewhere = std::max(slowest_elsewhere, t[i]);
-            if (best < 0 || t[i] < t[best]) best = i;
-        } else if (fastest_other == 0.f || t[i] < fastest_other) {
-            fastest_other = t[i];
-        }
+    std::vector<int> order;
+    try { order.reserve((size_t)n); } catch (const std::bad_alloc&) { return -1; }
+    for (int i = 0; i < n; ++i) if (t[i] > 0.f) order.push_back(i);           // a failed probe says nothing
+    if (order.empty()) return -1;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return t[a] < t[b]; });
+    const int best = order.front();
+    if (!spread_is_elsewhere(yardstick_ms, t[best])) return -1;               // nobody clearly below the yardstick
+    if (spread_is_elsewhere(yardstick_ms, t[order.back()])) return best;      // everybody is: the yardstick has spoken
+    // Two populations: somewhere among the times below the limit the sorted list must jump by kGap and more.  (The limit
+    // itself does not separate them: with a yardstick of 190 us it lies at 181 us, where candidates of the first
+    // allocation's own region have been seen -- 180.7 us in a search whose candidates elsewhere ended at 163 us.)
+    float widest = 0.f;
+    for (size_t k = 0; k + 1 < order.size(); ++k) {
+        const float lo = t[order[k]], hi = t[order[k + 1]];
+        if (!spread_is_elsewhere(yardstick_ms, lo)) break;
+        widest = std::max(widest, hi / lo - 1.f);
     }
-    if (best < 0) return -1;
-    // ... and the gap between the two populations, in the candidates' own times (every candidate elsewhere: nothing to compare with,
-    // the yardstick has spoken)
-    if (fastest_other > 0.f && fastest_other < (1.f + kGap) * slowest_elsewhere) return -1;
-    return best;
+    return widest >= kGap ? best : -1;
 }
 
 void pool_attach(int device, const void* owner) {

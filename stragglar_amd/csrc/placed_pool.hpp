@@ -33,9 +33,10 @@ struct SearchRecord {
 bool spread_yardstick(const float neighbours_ms[3], float ends_ms, float* yardstick_ms);
 // A single probe against the first allocation says "another region": clearly below the yardstick.
 bool spread_is_elsewhere(float yardstick_ms, float probe_ms);
-// All candidates' probe times at once: the index of the candidate to take (the fastest) when the times fall into two
-// populations -- candidates elsewhere, clearly below the yardstick, and the rest, with a clear gap between the two in
-// the candidates' own times --, else -1: nobody is clearly elsewhere, or the populations run into each other.
+// All candidates' probe times at once: the index of the candidate to take (the fastest) when it is clearly below the
+// yardstick and the times fall into two populations -- sorted, they jump by 4 % and more somewhere below the limit --,
+// or when every candidate is clearly below the yardstick; else -1: nobody is clearly elsewhere, or the times run on
+// without a gap.
 int spread_pick(float yardstick_ms, const float* probe_ms, int n);
 
 // ---- the pool ------------------------------------------------------------------------------------------------

@@ -612,6 +612,41 @@ def test_placed_memory_comes_back(sarlib, gpu_ctx):
     assert min(abs(after[0] - start), abs(after[0] - (start - pool_bytes))) <= slack, (start - after[0], pool_bytes)
 
 
+def test_a_step_behind_its_predecessor_gives_the_same_bits(sarlib, gpu_ctx, oracle):
+    """capi.Predecessor: the same schedule on a second set of rank buffers, run untimed before a timed step so that the
+    step starts with the caches as a sequence of AllReduces leaves them.  It must not touch the timed context's buffers:
+    twelve steps (the predecessor refills its own buffers every eighth), two dtypes, with and without pre-work, every
+    element against the checker each time the schedule changes."""
+    n = 8
+    for dtype, delay in (("f32", -1.0), ("bf16", 0.0)):
+        nbytes = sarlib.pad_bytes(1 << 20, n)
+        ctx = gpu_ctx
+        ctx.alloc_ranks(n, nbytes, dtype)
+        for r in range(n):
+            ctx.fill_uniform(r, 4200 + r, -1.0, 1.0)
+        ctx.snapshot()
+        inputs = [ctx.download(r) for r in range(n)]
+        main, pre = sarlib.parse(shipped_table(8), n), (sarlib.builtin("prework_rs", n) if delay >= 0 else None)
+        ctx.prepare(main, pre)
+        pred = ctx.predecessor(main, pre)
+        try:
+            assert (pred.ctx.n, pred.ctx.bytes_per_rank, pred.ctx.dtype) == (n, nbytes, dtype)
+            for _ in range(12):
+                ctx.restore()
+                pred.run(delay)
+                assert ctx.run(delay) > 0
+            whole_buffers_against_the_checker(ctx, oracle, "stragglar", inputs, dtype, read_golden("synth_pow2_n8.txt"), delay, "behind a predecessor")
+            ring = sarlib.builtin("ring", n)
+            ctx.prepare(ring, None)
+            pred.prepare(ring, None)
+            ctx.restore()
+            pred.run()
+            ctx.run(-1.0)
+            whole_buffers_against_the_checker(ctx, oracle, "ring", inputs, dtype, None, -1.0, "ring behind a predecessor")
+        finally:
+            pred.close()
+
+
 def test_contexts_share_the_placed_pair(sarlib, gpu_ctx, oracle):
     """Three contexts hold rank arenas on the GPU's one pair of placed allocations at the same time, and rows across its
     junction: leases do not overlap, every context computes the checker's bits whatever its neighbours do, the place

@@ -558,6 +558,16 @@ def test_region_search_decisions_on_recorded_probe_times(sarlib):
     assert sarlib.spread_pick(0.185, [0.190, 0.1739, 0.1813]) == 1
     assert sarlib.spread_pick(0.185, [0.1700]) == 0                                   # every candidate elsewhere: the yardstick has spoken
     assert sarlib.spread_pick(0.185, [0.1770]) == -1                                  # 0.957: not below the limit
+    # memory in which the regions alternate from candidate to candidate, and a candidate of the first allocation's region
+    # (180.7 us) just under the limit (0.95 x 190.5 = 181.0): the populations are 157.8-163.4 and 180.7-221.2, the jump
+    # between them is what counts, not on which side of the limit a candidate falls
+    y, _ = sarlib.spread_yardstick([0.1849, 0.1927, 0.1956], 0.1905)
+    mixed = [185.8, 159.5, 161.1, 159.5, 157.8, 161.4, 158.9, 157.9, 160.8, 158.2, 197.1, 161.8, 181.8, 158.6, 158.5, 160.1, 163.0, 180.7,
+             221.2, 159.7, 186.0, 158.5, 159.7, 159.9, 163.4]
+    assert sarlib.spread_pick(y, [t * 1e-3 for t in mixed]) == mixed.index(157.8)
+    # ... while times that run on without a jump are no verdict, wherever the limit cuts them
+    assert sarlib.spread_pick(0.200, [0.183, 0.186, 0.189, 0.192, 0.195, 0.199, 0.204]) == -1
+    assert sarlib.spread_pick(0.185, [0.150, 0.158, 0.163, 0.168, 0.173, 0.178, 0.183]) == 0        # the fastest stands clear of the rest
     # failed probes say nothing, and no candidates is no pair
     assert sarlib.spread_pick(0.185, [-1.0, 0.0, 0.158]) == 2
     assert sarlib.spread_pick(0.185, [-1.0]) == -1
