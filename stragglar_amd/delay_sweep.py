@@ -37,6 +37,7 @@ def main(argv=None) -> int:
     ap.add_argument("--delays", default="0,0.5,1,2,5")
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--algs", default="stragglar,ring,rhd,direct")
+    ap.add_argument("--behind-restore", action="store_true", help="no predecessor step: every timed run starts behind the restore alone")
     args = ap.parse_args(argv)
     lib = capi.load_library()
     n, dtype = args.ranks, args.dtype
@@ -49,7 +50,7 @@ def main(argv=None) -> int:
     for r in range(n):
         ctx.fill_uniform(r, 7 + r, -1.0, 1.0)
     ctx.snapshot()
-    pred = ctx.predecessor()
+    pred = None if args.behind_restore else ctx.predecessor()
     print("algorithm,buffer_size_bytes,delay,runtime_ms,runtime_minus_delay_ms,BW(GB/s)")
     net = {}
     for alg in algs:
@@ -63,12 +64,14 @@ def main(argv=None) -> int:
             main_sched = lib.builtin(alg, n)
             prework = lib.builtin("prework_ar", n) if alg == "direct" else None
         ctx.prepare(main_sched, prework)
-        pred.prepare(main_sched, prework)
+        if pred:
+            pred.prepare(main_sched, prework)
         for d in delays:
             ts = []
             for it in range(args.iters + 1):
                 ctx.restore()
-                pred.run(d)
+                if pred:
+                    pred.run(d)
                 ms = ctx.run(d)
                 if it:
                     ts.append(ms)
@@ -76,7 +79,8 @@ def main(argv=None) -> int:
             rest = ms - (d if d > 0 else 0.0)
             net[(alg, d)] = rest
             print("%s,%d,%.3f,%.3f,%.3f,%.3f" % (alg, nbytes, d, ms, rest, nbytes / 2 ** 30 * 1000 / rest))
-    pred.close()
+    if pred:
+        pred.close()
     ctx.close()
     if "ring" in algs:
         print("# milliseconds saved against ring after the straggler has arrived (positive = finishes sooner)")

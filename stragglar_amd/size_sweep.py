@@ -37,6 +37,7 @@ def main(argv=None) -> int:
     ap.add_argument("--sizes", default="4096,65536,1048576,16777216,268435456,1073741824")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--algs", default="stragglar,ring,rhd,direct")
+    ap.add_argument("--behind-restore", action="store_true", help="no predecessor step: every timed run starts behind the restore alone")
     args = ap.parse_args(argv)
     lib = capi.load_library()
     n = args.ranks
@@ -48,7 +49,7 @@ def main(argv=None) -> int:
         for r in range(n):
             ctx.fill_uniform(r, 11 + r, -1.0, 1.0)
         ctx.snapshot()
-        pred = ctx.predecessor()
+        pred = None if args.behind_restore else ctx.predecessor()
         for alg in [a for a in args.algs.split(",") if a]:
             if alg == "stragglar":
                 path = os.path.join(HERE, "schedules", "stragglar_n%d.txt" % n)
@@ -59,12 +60,14 @@ def main(argv=None) -> int:
                 sched = lib.builtin(alg, n)
             for graph in (0, 1):
                 ctx.prepare(sched, None, use_graph=bool(graph))
-                pred.prepare(sched, None)
+                if pred:
+                    pred.prepare(sched, None)
                 st = ctx.stats()
                 ts, host = [], []
                 for it in range(args.iters + 2):
                     ctx.restore()
-                    pred.run()
+                    if pred:
+                        pred.run()
                     t0 = time.perf_counter()
                     ms = ctx.run(-1.0)
                     t1 = time.perf_counter()
@@ -76,7 +79,8 @@ def main(argv=None) -> int:
                 print("%s,%d,%d,%d,%s,%.2f,%.2f,%.0f,%.0f,%.1f" % (alg, nbytes, graph, st.launches, "column" if st.executor else "rounds",
                                                                   med * 1e3, min(ts) * 1e3, to_memory / med / 1e6, st.algorithmic_bytes / med / 1e6,
                                                                   statistics.median(host) * 1e6), flush=True)
-        pred.close()                          # before the next size: both sets of rank buffers lease from one pool
+        if pred:
+            pred.close()                      # before the next size: both sets of rank buffers lease from one pool
     ctx.close()
     return 0
 
