@@ -414,7 +414,7 @@ private:
         // Nothing is read twice and every row is a pairwise row (the exchanges of a table on their own): nothing to keep in
         // slots, two cold loads and one or two stores per vector, and the narrower column runs ahead (n = 8, in a sequence
         // of steps: 256 MiB per rank 172.8 against 175.0 us, 1 GiB 681 against 698).  A plan of multi-source rows alone
-        // (a pre-work) is the other way round: 1024 > 512 > 256 threads by 1 - 2 % each.
+        // (a pre-work) stays at 512: 1024 threads gain 1.7 % at 1 GiB fp32 per rank, nothing in bf16 and lose 2.5 % at 256 MiB.
         if (no_reuse_ && !env_.tune.col_block && !plan_.staged && plan_.block == 512) {
             bool pairwise = !cr_.empty();
             for (const auto& r : cr_) pairwise = pairwise && r.d.kind != SAR_OP_MREDUCE;
