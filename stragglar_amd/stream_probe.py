@@ -18,6 +18,8 @@ counted -- moves the same bytes between the same addresses as
                 rank's copy is read once and written once (n reads + n writes in place)
     direct      the same for direct: rank 0's and the straggler's whole buffers are read, the sum goes to every rank
     copy/read/write   one buffer copied to another; all buffers read; all buffers written
+    runtime_copy      not the probe: the runtime's own device-to-device copy (hipMemcpyAsync) of every rank buffer, one after the
+                      other, timed on the host clock around the synchronising call -- a yardstick that nobody here wrote
 
 With 16, 24, ... 64 ranks (--ranks) the mixes are instead
 
@@ -98,6 +100,19 @@ def main(argv=None) -> int:
         print("%s,%d x (%dR+%dW),%d,%.1f,%.0f,%.3f,%d/%d/%d/%d/%d,%.1f,%d"
               % (name, len(jobs), len(rd), len(wr), res.bytes_moved, res.best_ms * 1e3, res.gbps, res.gbps / PEAK,
                  res.block, res.unroll, res.nontemporal, res.persistent, res.interleave, res.worst_ms * 1e3, res.variants), flush=True)
+    if n <= 8 and (not want or "runtime_copy" in want):
+        # a yardstick nobody here wrote: the runtime's own device-to-device copy (hipMemcpyAsync, which sar_snapshot
+        # uses), every rank buffer to its snapshot one after the other, on the host clock around the synchronising call
+        import time
+        ctx.snapshot()                                          # allocates the snapshot
+        best = None
+        for _ in range(max(2, args.reps)):
+            t0 = time.perf_counter()
+            ctx.snapshot()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        moved = 2 * n * nbytes
+        print("runtime_copy,%d x (1R+1W),%d,%.1f,%.0f,%.3f,hipMemcpyAsync,%.1f,1" % (n, moved, best * 1e6, moved / best / 1e9, moved / best / 1e9 / PEAK, best * 1e6), flush=True)
     ctx.close()
     return 0
 

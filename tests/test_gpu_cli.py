@@ -172,8 +172,9 @@ def test_measurement_tools_run():
     p = run(sys.executable, "-m", "stragglar_amd.stream_probe", "--mib", "4", "--reps", "1")
     assert p.returncode == 0, p.stdout + p.stderr
     rows = [l.split(",") for l in p.stdout.splitlines()[2:]]
-    assert [r[0] for r in rows] == ["exchanges", "one", "schedule", "prework", "ring", "direct", "copy", "read", "write"]
+    assert [r[0] for r in rows] == ["exchanges", "one", "schedule", "prework", "ring", "direct", "copy", "read", "write", "runtime_copy"]
     assert all(len(r) == 9 and float(r[3]) > 0 and float(r[4]) > 0 for r in rows)
+    assert rows[-1][1] == "8 x (1R+1W)" and rows[-1][6] == "hipMemcpyAsync"
     assert rows[2][1] == "7 x (2R+8W)" and int(rows[2][2]) * 4 == int(rows[0][2]) * 10         # 10 streams a job against 4
     # more than eight ranks: every buffer read and written once by jobs of eight ranks each
     p = run(sys.executable, "-m", "stragglar_amd.stream_probe", "--ranks", "16", "--mib", "2", "--reps", "1")
