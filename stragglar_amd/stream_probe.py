@@ -28,6 +28,9 @@ With 16, 24, ... 64 ranks (--ranks) the mixes are instead
     eights_strided  the same with job j on ranks j, j + n/8, ... (half of them in either region of HBM)
 
 One line per mix: microseconds, GB/s, fraction of the 8 TB/s peak, the fastest shape and the slowest shape's time.
+
+--torch runs none of this but PyTorch's own elementwise kernels (copy_, add_, add with out=, fill_, sum) on fp32 tensors
+of one and of n rank buffers' size: what kernels by other authors reach on the same chip.
 """
 import argparse
 import sys
@@ -61,6 +64,39 @@ def mixes_many(n, whole):
             ("eights_strided", [(list(range(j, n, g)), list(range(j, n, g)), 0) for j in range(g)], whole)]
 
 
+def torch_rates(args) -> int:
+    """PyTorch's elementwise kernels as a yardstick from outside this code: fastest and median of ten runs, timed with
+    torch's events on torch's stream; fp32 tensors in one ordinary allocation each."""
+    import torch
+    if not torch.cuda.is_available():
+        print("--torch needs a GPU that torch can see", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    print("tensor_bytes,operation,streams,bytes_moved,min_us,median_us,GB/s(min),frac_of_8TBps")
+    for nbytes in (int(args.mib * (1 << 20)), int(args.mib * (1 << 20)) * args.ranks):
+        elems = nbytes // 4
+        a, b, c = torch.rand(elems, device=dev), torch.rand(elems, device=dev), torch.empty(elems, device=dev)
+        for name, streams, fn, moved in (("c.copy_(a)", "1R+1W", lambda: c.copy_(a), 2), ("a.add_(b)", "2R+1W", lambda: a.add_(b), 3),
+                                         ("torch.add(a b out=c)", "2R+1W", lambda: torch.add(a, b, out=c), 3),
+                                         ("c.fill_(1.0)", "0R+1W", lambda: c.fill_(1.0), 1), ("a.sum()", "1R+0W", lambda: a.sum(), 1)):
+            fn()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(10):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                e1.synchronize()
+                ts.append(e0.elapsed_time(e1))
+            ts.sort()
+            bytes_moved = moved * elems * 4
+            print("%d,%s,%s,%d,%.1f,%.1f,%.0f,%.3f" % (elems * 4, name, streams, bytes_moved, ts[0] * 1e3, ts[len(ts) // 2] * 1e3,
+                                                      bytes_moved / ts[0] / 1e6, bytes_moved / ts[0] / 1e6 / PEAK), flush=True)
+        del a, b, c
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--ranks", type=int, default=8)
@@ -69,7 +105,11 @@ def main(argv=None) -> int:
     ap.add_argument("--reps", type=int, default=5)
     ap.add_argument("--spread", type=int, default=1, choices=[0, 1], help="0 = all rank buffers back to back in one allocation")
     ap.add_argument("--mix", default="", help="comma-separated subset of the mixes")
+    ap.add_argument("--torch", action="store_true", help="instead of the probe: PyTorch's own elementwise kernels on tensors of one and of n rank buffers' size "
+                    "(copy_, add_, add with out=, fill_, sum) -- what other authors' kernels reach on the same chip")
     args = ap.parse_args(argv)
+    if args.torch:
+        return torch_rates(args)
     lib = capi.load_library()
     n = args.ranks
     if n < 3 or (n > 8 and (n % 8 or n > 64)):

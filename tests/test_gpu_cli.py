@@ -183,6 +183,10 @@ def test_measurement_tools_run():
     assert [r[0] for r in rows] == ["eights", "eights_strided"] and all(r[1] == "2 x (8R+8W)" for r in rows)
     per_rank = int(p.stdout.splitlines()[0].split(",")[1].split()[0])
     assert all(int(r[2]) == 2 * 16 * per_rank and float(r[4]) > 0 for r in rows)
+    p = run(sys.executable, "-m", "stragglar_amd.stream_probe", "--torch", "--mib", "8")
+    assert p.returncode == 0, p.stdout + p.stderr
+    rows = [l.split(",") for l in p.stdout.splitlines()[1:]]
+    assert len(rows) == 10 and all(float(r[4]) > 0 and float(r[6]) > 0 for r in rows)
     p = run(sys.executable, "-m", "stragglar_amd.stream_probe", "--ranks", "12")
     assert p.returncode == 2 and "16, 24, ... 64" in p.stderr
     p = run(sys.executable, "-m", "stragglar_amd.hbm_regions", "--gib", "16", "--slot-gib", "1", "--stream-mib", "8", "--reps", "1")
