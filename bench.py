@@ -202,6 +202,19 @@ class Steps:
         if self.pred is not None:
             self.pred.run(delay)          # untimed: the step before this one, on buffers of its own
 
+    def behind_restore(self, steps, delay=-1.0):
+        """Mean of `steps` steps timed behind the restore alone, for the record of what the predecessor changes (one untimed
+        step first); None when that is how all steps of this run are timed anyway."""
+        if self.pred is None:
+            return None
+        out = []
+        for i in range(steps + 1):
+            self.ctx.restore()
+            ms = self.ctx.run(delay)
+            if i:
+                out.append(ms)
+        return round(statistics.fmean(out), 5)
+
     def timed(self, steps, warmup, delay=-1.0):
         for _ in range(warmup):
             self.ready(delay)
@@ -422,6 +435,7 @@ def main():
         ctx.close()
         return
     ms = statistics.fmean(step_ms)
+    clean_ms = seq.behind_restore(max(3, args.steps // 2))
     # the same K steps back to back on the host clock, no restore in between (the sums just keep growing):
     # a cross-check of the event timing that includes launch and synchronisation overhead
     ctx.restore()
@@ -497,6 +511,8 @@ def main():
         # stores of values that a later row overwrites before anybody loads them (none in the StragglAR tables)
         "elided_store_bytes_per_step": int(st.elided_store_bytes),
         "ms_per_step_min": round(min(step_ms), 5),
+        # the same steps timed behind the restore alone (clean Infinity Cache, no step in front): what the step protocol changes
+        "ms_per_step_behind_restore": clean_ms,
         "wall_ms_per_step_back_to_back": round(back_to_back_ms, 4),
         "ranks_identical_after_run": bool(identical),
         # 1 = the two halves of the rank buffers were placed in different regions of HBM (sar_alloc_ranks)
@@ -550,7 +566,8 @@ def main():
         xm = statistics.fmean(xms)
         xmem, xhbm, _ = rates(xst, xm)
         rec["reduce_steps_alone"] = {"rows": "%d exchanges (XREDUCE) of one chunk each, no copies" % (n - 1), "ms_per_step": round(xm, 5),
-                                     "ms_per_step_min": round(min(xms), 5), "memory_bytes_per_step": int(xmem),
+                                     "ms_per_step_min": round(min(xms), 5), "ms_per_step_behind_restore": seq.behind_restore(max(3, args.steps // 2)),
+                                     "memory_bytes_per_step": int(xmem),
                                      "GBps": round(xhbm, 1), "frac_of_hbm_peak": round(xhbm / HBM_PEAK_GBPS, 4),
                                      "executor_used": "column" if xst.executor == 1 else "rounds", "launches": int(xst.launches)}
         if 2 <= n - 1 <= 8:
@@ -606,7 +623,7 @@ def main():
             cms = seq.timed(args.steps, args.warmup)
             cm = statistics.fmean(cms)
             cmem, chbm, calg = rates(cst, cm)
-            leg = {"ms_per_step": round(cm, 5), "ms_per_step_min": round(min(cms), 5),
+            leg = {"ms_per_step": round(cm, 5), "ms_per_step_min": round(min(cms), 5), "ms_per_step_behind_restore": seq.behind_restore(max(3, args.steps // 2)),
                    "memory_side_GBps": round(chbm, 1), "frac_of_hbm_peak": round(chbm / HBM_PEAK_GBPS, 4),
                    "memory_bytes_per_step": int(cmem), "algorithmic_bytes_per_step": int(cst.algorithmic_bytes),
                    "algorithmic_GBps": round(calg, 1), "executor_used": "column" if cst.executor == 1 else "rounds",

@@ -265,6 +265,7 @@ def test_bench_prints_one_json_line_with_the_agreed_keys(extra):
     assert abs(roof["achieved"] - roof["memory_bytes_per_launch"] / roof["mean_launch_ms"] / 1e6) <= 0.002 * roof["achieved"]
     assert rec["host"]["logical_cpus"] >= 1
     assert ("restore alone" in rec["config"]["timed"]) == ("--behind-restore" in extra)
+    assert (rec["ms_per_step_behind_restore"] is None) == ("--behind-restore" in extra)
     if "--no-live-traffic" not in extra:
         import shutil
         if shutil.which("rocprofv3"):
